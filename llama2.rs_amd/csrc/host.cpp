@@ -1,0 +1,1102 @@
+// Host side of the C ABI: checkpoint loading and upload (LlamaModel::from_file,
+// src/lib.rs:45-104), RunState (src/models.rs:29-42), the layer schedule of
+// transformer<B> (src/models.rs:178-298) and the greedy loop of generate
+// (src/inference.rs:16-193), driving the HIP kernels.  Nothing here computes on
+// the CPU except the one-time RoPE angle table and the synthetic-image
+// generator.
+#include <fcntl.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <chrono>
+#include <numeric>
+#include <thread>
+
+#include "l2_internal.h"
+
+// ---------------------------------------------------------------------------
+// errors
+
+static thread_local char g_err[512] = "";
+
+int l2_fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+extern "C" const char *l2_last_error(void) { return g_err; }
+
+// ---------------------------------------------------------------------------
+// dims, presets, sizes
+
+static int64_t div_up(int64_t x, int64_t y) { return x / y + (x % y == 0 ? 0 : 1); }
+
+static size_t qlinear_bytes(int in, int out, int g) {
+    const size_t groups = (size_t)div_up(in, g);
+    return (size_t)out * (in / 8) * 4 + (size_t)(out / 8) * groups * 4 + (size_t)out * groups * 4 +
+           (size_t)in * 4;
+}
+
+static int check_dims(const l2_dims *d) {
+    if (!d) return l2_fail(L2_ERR_ARG, "dims is null");
+    if (d->dim <= 0 || d->hidden_dim <= 0 || d->n_layers <= 0 || d->n_heads <= 0 ||
+        d->n_kv_heads <= 0 || d->vocab_size <= 0 || d->seq_len <= 0)
+        return l2_fail(L2_ERR_ARG, "dims: non-positive field");
+    if (d->group_size != 32 && d->group_size != 64 && d->group_size != 128)
+        return l2_fail(L2_ERR_ARG, "dims: group_size %d (32, 64 or 128)", d->group_size);
+    if (d->dim % d->n_heads || d->n_heads % d->n_kv_heads)
+        return l2_fail(L2_ERR_ARG, "dims: heads do not divide");
+    if (d->dim / d->n_heads != 128)
+        return l2_fail(L2_ERR_ARG, "dims: head size %d (the kernels are built for 128)", d->dim / d->n_heads);
+    if (d->dim % d->group_size || d->hidden_dim % d->group_size || d->dim % 32 || d->hidden_dim % 32)
+        return l2_fail(L2_ERR_ARG, "dims: dim and hidden_dim must be multiples of 32 and of the group size");
+    return L2_OK;
+}
+
+extern "C" int l2_preset(const char *model_size, int group_size, l2_dims *out) {
+    if (!model_size || !out) return l2_fail(L2_ERR_ARG, "l2_preset: null argument");
+    l2_dims d;
+    // src/constants.rs:7-41
+    if (!strcmp(model_size, "7B"))
+        d = {4096, 11008, 32, 32, 32, 32000, 2048, group_size};
+    else if (!strcmp(model_size, "13B"))
+        d = {5120, 13824, 40, 40, 40, 32000, 2048, group_size};
+    else if (!strcmp(model_size, "70B"))
+        d = {8192, 28672, 80, 64, 8, 32000, 2048, group_size};
+    else
+        return l2_fail(L2_ERR_ARG, "l2_preset: model size '%s' (7B, 13B or 70B)", model_size);
+    L2_TRY(check_dims(&d));
+    *out = d;
+    return L2_OK;
+}
+
+extern "C" size_t l2_weights_bytes(const l2_dims *d) {
+    if (!d || d->n_heads <= 0) return 0;
+    const int hs = d->dim / d->n_heads;
+    const int kv_dim = d->n_kv_heads * hs;
+    const size_t L = (size_t)d->n_layers;
+    const int G = d->group_size;
+    size_t n = 4;
+    n += (size_t)d->vocab_size * d->dim * 4;
+    n += L * d->dim * 4;
+    n += L * (2 * qlinear_bytes(d->dim, d->dim, G) + 2 * qlinear_bytes(d->dim, kv_dim, G));
+    n += L * d->dim * 4;
+    n += L * (2 * qlinear_bytes(d->dim, d->hidden_dim, G) + qlinear_bytes(d->hidden_dim, d->dim, G));
+    n += (size_t)d->dim * 4;
+    n += (size_t)d->seq_len * (hs / 2) * 4 * 2;
+    n += (size_t)d->vocab_size * d->dim * 4;
+    return n;
+}
+
+// ---------------------------------------------------------------------------
+// synthetic image
+
+namespace {
+
+struct Rng { // splitmix64
+    uint64_t s;
+    explicit Rng(uint64_t seed) : s(seed) {}
+    uint64_t next() {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    double uniform() { return (double)(next() >> 11) * (1.0 / 9007199254740992.0); }
+    float normal(float sigma) {
+        double u1 = uniform(), u2 = uniform();
+        if (u1 < 1e-300) u1 = 1e-300;
+        return (float)(sigma * sqrt(-2.0 * log(u1)) * cos(6.283185307179586 * u2));
+    }
+};
+
+// One tensor-sized job of the generator; jobs are independent so that threads
+// can take them in any order and still produce the same bytes.
+struct SynthJob {
+    char *dst;
+    size_t n; // elements
+    int kind; // 0 random words, 1 scales, 2 normal(0.02), 3 g_index, 4 freq cos, 5 freq sin
+    uint64_t seed;
+    int a, b; // g_index: in, group_size; freq: seq_len, half
+};
+
+void run_job(const SynthJob &j) {
+    Rng r(j.seed);
+    switch (j.kind) {
+        case 0: {
+            uint32_t *p = (uint32_t *)j.dst;
+            size_t i = 0;
+            for (; i + 1 < j.n; i += 2) {
+                const uint64_t v = r.next();
+                p[i] = (uint32_t)v;
+                p[i + 1] = (uint32_t)(v >> 32);
+            }
+            if (i < j.n) p[i] = (uint32_t)r.next();
+            break;
+        }
+        case 1: {
+            float *p = (float *)j.dst;
+            for (size_t i = 0; i < j.n; i++) p[i] = (float)(0.002 + 0.018 * r.uniform());
+            break;
+        }
+        case 2: {
+            float *p = (float *)j.dst;
+            for (size_t i = 0; i < j.n; i++) p[i] = r.normal(0.02f);
+            break;
+        }
+        case 3: {
+            // g_idx = shuffled i / group_size; g_index = stable argsort(g_idx)
+            // (export.py:52,65)
+            const int in = j.a, G = j.b;
+            std::vector<int32_t> gidx(in);
+            for (int i = 0; i < in; i++) gidx[i] = i / G;
+            for (int i = in - 1; i > 0; i--) {
+                const int k = (int)(r.next() % (uint64_t)(i + 1));
+                std::swap(gidx[i], gidx[k]);
+            }
+            const int groups = (in + G - 1) / G;
+            std::vector<int32_t> start(groups + 1, 0);
+            for (int i = 0; i < in; i++) start[gidx[i] + 1]++;
+            for (int g = 0; g < groups; g++) start[g + 1] += start[g];
+            int32_t *p = (int32_t *)j.dst;
+            for (int i = 0; i < in; i++) p[start[gidx[i]]++] = i;
+            break;
+        }
+        case 4:
+        case 5: {
+            float *p = (float *)j.dst;
+            const int half = j.b;
+            for (int t = 0; t < j.a; t++)
+                for (int i = 0; i < half; i++) {
+                    const float f = 1.0f / powf(10000.0f, (float)(2 * i) / (float)(2 * half));
+                    const float ang = (float)t * f;
+                    p[(size_t)t * half + i] = j.kind == 4 ? cosf(ang) : sinf(ang);
+                }
+            break;
+        }
+    }
+}
+
+// Walk the image in struct order (src/gptq.rs:34-84), calling f(kind, ptr, elems, in, out).
+struct Walker {
+    const l2_dims &d;
+    char *p;
+    std::vector<SynthJob> jobs;
+    uint64_t seed;
+    uint64_t counter = 0;
+    void add(int kind, size_t n, int a = 0, int b = 0) {
+        // big tensors are cut into slices so that the threads stay balanced
+        const size_t slice = (kind == 3 || kind == 4 || kind == 5) ? n : ((size_t)1 << 22);
+        for (size_t off = 0; off < n; off += slice) {
+            const size_t m = std::min(slice, n - off);
+            jobs.push_back({p + off * 4, m, kind, seed * 0x100000001B3ull + (++counter) * 0x9E3779B97F4A7C15ull, a, b});
+        }
+        p += n * 4;
+    }
+    void qlinears(int in, int out) {
+        const int G = d.group_size;
+        const size_t groups = (size_t)div_up(in, G);
+        for (int l = 0; l < d.n_layers; l++) {
+            add(0, (size_t)out * (in / 8));
+            add(0, (size_t)(out / 8) * groups);
+            add(1, (size_t)out * groups);
+            add(3, (size_t)in, in, G);
+        }
+    }
+};
+
+} // namespace
+
+extern "C" int l2_synth_image(const l2_dims *d, uint64_t seed, void *buf, size_t nbytes) {
+    L2_TRY(check_dims(d));
+    if (!buf) return l2_fail(L2_ERR_ARG, "l2_synth_image: null buffer");
+    if (nbytes != l2_weights_bytes(d))
+        return l2_fail(L2_ERR_ARG, "l2_synth_image: buffer is %zu bytes, image is %zu", nbytes, l2_weights_bytes(d));
+    const int hs = d->dim / d->n_heads, kv_dim = d->n_kv_heads * hs;
+    Walker w{*d, (char *)buf, {}, seed};
+    const float eps = 1e-5f;
+    memcpy(w.p, &eps, 4);
+    w.p += 4;
+    w.add(2, (size_t)d->vocab_size * d->dim);
+    w.add(2, (size_t)d->n_layers * d->dim);
+    w.qlinears(d->dim, d->dim);
+    w.qlinears(d->dim, kv_dim);
+    w.qlinears(d->dim, kv_dim);
+    w.qlinears(d->dim, d->dim);
+    w.add(2, (size_t)d->n_layers * d->dim);
+    w.qlinears(d->dim, d->hidden_dim);
+    w.qlinears(d->hidden_dim, d->dim);
+    w.qlinears(d->dim, d->hidden_dim);
+    w.add(2, (size_t)d->dim);
+    w.add(4, (size_t)d->seq_len * (hs / 2), d->seq_len, hs / 2);
+    w.add(5, (size_t)d->seq_len * (hs / 2), d->seq_len, hs / 2);
+    w.add(2, (size_t)d->vocab_size * d->dim);
+    if ((size_t)(w.p - (char *)buf) != nbytes) return l2_fail(L2_ERR_ARG, "l2_synth_image: internal size mismatch");
+    unsigned nt = std::thread::hardware_concurrency();
+    if (nt == 0) nt = 1;
+    if (nt > 16) nt = 16;
+    std::vector<std::thread> th;
+    for (unsigned t = 0; t < nt; t++)
+        th.emplace_back([&, t]() {
+            for (size_t i = t; i < w.jobs.size(); i += nt) run_job(w.jobs[i]);
+        });
+    for (auto &t : th) t.join();
+    return L2_OK;
+}
+
+// ---------------------------------------------------------------------------
+// model
+
+struct l2_model {
+    l2_dims d{};
+    l2_config cfg{};
+    int max_seq = 0;
+    int head_size = 0, kv_dim = 0;
+    float rms_eps = 0.f;
+    int prefill_mode = L2_PREFILL_FP32;
+    hipStream_t stream = nullptr;
+
+    char *dimage = nullptr; // device copy of the weights image (shifted to 128-byte alignment)
+    const float *tok_emb = nullptr, *rms_att = nullptr, *rms_ffn = nullptr, *rms_final = nullptr,
+                *wcls = nullptr;
+    std::vector<DevQLinear> q[7]; // indexed by L2_WQ..L2_W3, then layer
+    int32_t *dinv = nullptr;      // all inverse permutations
+    float *rope_cos = nullptr, *rope_sin = nullptr; // [max_seq][head_size/2]
+
+    // forward scratch, sized for cap_B batch columns
+    int cap_B = 0;
+    float *x = nullptr, *xq = nullptr, *xk = nullptr, *xv = nullptr, *qv = nullptr, *kv = nullptr,
+          *vv = nullptr, *attg = nullptr, *x1 = nullptr, *x3 = nullptr, *hb = nullptr, *hb2 = nullptr,
+          *hg = nullptr, *fin = nullptr, *logits = nullptr;
+    int32_t *dtok = nullptr, *dpos = nullptr;
+    unsigned long long *amax = nullptr;
+    int32_t *dprompt = nullptr, *dout_ids = nullptr;
+    int cap_prompt = 0, cap_out = 0;
+    // scratch for the operator-level entry points
+    float *op_x = nullptr, *op_xg = nullptr, *op_y = nullptr;
+    size_t op_cap = 0;
+};
+
+struct l2_state {
+    l2_model *m = nullptr;
+    float *kcache = nullptr, *vcache = nullptr; // [L][max_seq][kv_dim]
+    size_t elems = 0;
+};
+
+struct l2_qlinear {
+    DevQLinear q;
+    void *bufs[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    hipStream_t stream = nullptr;
+    float *x = nullptr, *xg = nullptr, *y = nullptr;
+    int cap_B = 0;
+};
+
+extern "C" int l2_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+static int require_device() {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n < 1) {
+        (void)hipGetLastError();
+        return l2_fail(L2_ERR_HIP, "no HIP device available (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    }
+    return L2_OK;
+}
+
+template <typename T>
+static int dalloc(T **p, size_t n) {
+    void *v = nullptr;
+    hipError_t e = hipMalloc(&v, n * sizeof(T) ? n * sizeof(T) : 16);
+    if (e != hipSuccess) return l2_fail(L2_ERR_HIP, "hipMalloc(%zu bytes): %s", n * sizeof(T), hipGetErrorString(e));
+    *p = (T *)v;
+    return L2_OK;
+}
+
+static void dfree(void *p) {
+    if (p) (void)hipFree(p);
+}
+
+static void invert_perm(const int32_t *g, int n, int32_t *inv, bool *ok) {
+    std::fill(inv, inv + n, -1);
+    for (int j = 0; j < n; j++) {
+        const int32_t v = g[j];
+        if (v < 0 || v >= n || inv[v] != -1) {
+            *ok = false;
+            return;
+        }
+        inv[v] = j;
+    }
+}
+
+static constexpr size_t kImageShift = 124; // image offset 4 (first tensor) lands on a 128-byte boundary
+
+static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, int max_seq, l2_model **out) {
+    L2_TRY(check_dims(dims));
+    if (!weights || !out) return l2_fail(L2_ERR_ARG, "null argument");
+    if (nbytes != l2_weights_bytes(dims)) // src/lib.rs:97
+        return l2_fail(L2_ERR_FORMAT, "weights are %zu bytes, the struct for these dims is %zu", nbytes,
+                       l2_weights_bytes(dims));
+    if (max_seq <= 0) max_seq = dims->seq_len;
+    if (max_seq > 15000) return l2_fail(L2_ERR_RANGE, "max_seq %d (at most 15000)", max_seq);
+    L2_TRY(require_device());
+
+    l2_model *m = new l2_model();
+    m->d = *dims;
+    m->max_seq = max_seq;
+    m->head_size = dims->dim / dims->n_heads;
+    m->kv_dim = dims->n_kv_heads * m->head_size;
+    m->cfg = {dims->dim, dims->hidden_dim, dims->n_layers, dims->n_heads, dims->n_kv_heads,
+              dims->vocab_size, dims->seq_len, 0};
+    auto bail = [&](int rc) {
+        l2_model_close(m);
+        return rc;
+    };
+#define M_HIP(call)                                                                              \
+    do {                                                                                         \
+        hipError_t e_ = (call);                                                                  \
+        if (e_ != hipSuccess)                                                                    \
+            return bail(l2_fail(L2_ERR_HIP, "%s: %s", #call, hipGetErrorString(e_)));            \
+    } while (0)
+#define M_TRY(call)                    \
+    do {                               \
+        int rc_ = (call);              \
+        if (rc_ != L2_OK) return bail(rc_); \
+    } while (0)
+
+    M_HIP(hipStreamCreate(&m->stream));
+    M_TRY(dalloc(&m->dimage, nbytes + 256));
+    char *dbase = m->dimage + kImageShift;
+    // one pass over the host image, in 64 MiB pieces so that a mapped file is paged in as it goes
+    for (size_t off = 0; off < nbytes; off += (size_t)64 << 20) {
+        const size_t n = std::min((size_t)64 << 20, nbytes - off);
+        M_HIP(hipMemcpy(dbase + off, weights + off, n, hipMemcpyHostToDevice));
+    }
+
+    // views, in struct order (src/gptq.rs:34-66)
+    const int L = dims->n_layers, G = dims->group_size, dim = dims->dim, hid = dims->hidden_dim;
+    size_t off = 0;
+    memcpy(&m->rms_eps, weights, 4);
+    off += 4;
+    auto f32 = [&](size_t n) {
+        const float *p = (const float *)(dbase + off);
+        off += n * 4;
+        return p;
+    };
+    size_t inv_total = 0;
+    struct Pending { int proj, layer; size_t host_off; int in; size_t inv_off; };
+    std::vector<Pending> pend;
+    auto qblock = [&](int proj, int in, int outn) {
+        const int groups = (int)div_up(in, G);
+        m->q[proj].resize(L);
+        for (int l = 0; l < L; l++) {
+            DevQLinear &q = m->q[proj][l];
+            q.in = in;
+            q.out = outn;
+            q.groups = groups;
+            q.group_size = G;
+            q.qweight = (const uint4 *)(dbase + off);
+            off += (size_t)outn * (in / 8) * 4;
+            q.qzeros = (const int32_t *)(dbase + off);
+            off += (size_t)(outn / 8) * groups * 4;
+            q.scales = (const float *)(dbase + off);
+            off += (size_t)outn * groups * 4;
+            q.g_index = (const int32_t *)(dbase + off);
+            pend.push_back({proj, l, off, in, inv_total});
+            inv_total += (size_t)in;
+            off += (size_t)in * 4;
+        }
+    };
+    m->tok_emb = f32((size_t)dims->vocab_size * dim);
+    m->rms_att = f32((size_t)L * dim);
+    qblock(L2_WQ, dim, dim);
+    qblock(L2_WK, dim, m->kv_dim);
+    qblock(L2_WV, dim, m->kv_dim);
+    qblock(L2_WO, dim, dim);
+    m->rms_ffn = f32((size_t)L * dim);
+    qblock(L2_W1, dim, hid);
+    qblock(L2_W2, hid, dim);
+    qblock(L2_W3, dim, hid);
+    m->rms_final = f32((size_t)dim);
+    off += (size_t)dims->seq_len * (m->head_size / 2) * 4 * 2; // deprecated tables, never read (src/models.rs:193-197)
+    m->wcls = f32((size_t)dims->vocab_size * dim);
+    if (off != nbytes) return bail(l2_fail(L2_ERR_FORMAT, "internal: walked %zu of %zu bytes", off, nbytes));
+
+    // inverse act-order permutations (also validates every g_index)
+    {
+        std::vector<int32_t> inv(inv_total);
+        bool ok = true;
+        for (const Pending &p : pend) {
+            invert_perm((const int32_t *)(weights + p.host_off), p.in, inv.data() + p.inv_off, &ok);
+            if (!ok)
+                return bail(l2_fail(L2_ERR_FORMAT, "g_index of projection %d, layer %d is not a permutation of 0..%d",
+                                    p.proj, p.layer, p.in - 1));
+        }
+        M_TRY(dalloc(&m->dinv, inv_total));
+        M_HIP(hipMemcpy(m->dinv, inv.data(), inv_total * 4, hipMemcpyHostToDevice));
+        for (const Pending &p : pend) m->q[p.proj][p.layer].inv_index = m->dinv + p.inv_off;
+    }
+
+    // RoPE angles exactly as the reference evaluates them per element
+    // (src/models.rs:107-110), computed once with the host's libm.
+    {
+        const int half = m->head_size / 2;
+        std::vector<float> c((size_t)max_seq * half), s((size_t)max_seq * half);
+        for (int i = 0; i < half; i++) {
+            const float freq = 1.0f / powf(10000.0f, ((float)((2 * i) % m->head_size)) / (float)m->head_size);
+            for (int p = 0; p < max_seq; p++) {
+                const float val = (float)p * freq;
+                c[(size_t)p * half + i] = cosf(val);
+                s[(size_t)p * half + i] = sinf(val);
+            }
+        }
+        M_TRY(dalloc(&m->rope_cos, c.size()));
+        M_TRY(dalloc(&m->rope_sin, s.size()));
+        M_HIP(hipMemcpy(m->rope_cos, c.data(), c.size() * 4, hipMemcpyHostToDevice));
+        M_HIP(hipMemcpy(m->rope_sin, s.data(), s.size() * 4, hipMemcpyHostToDevice));
+    }
+    M_TRY(dalloc(&m->amax, 1));
+    M_HIP(hipDeviceSynchronize());
+#undef M_HIP
+#undef M_TRY
+    *out = m;
+    return L2_OK;
+}
+
+extern "C" int l2_model_from_image(const void *weights, size_t nbytes, const l2_dims *dims, int max_seq,
+                                   l2_model **out) {
+    return model_build((const char *)weights, nbytes, dims, max_seq, out);
+}
+
+extern "C" int l2_model_open(const char *path, const l2_dims *expect, int max_seq, l2_model **out) {
+    if (!path || !expect || !out) return l2_fail(L2_ERR_ARG, "l2_model_open: null argument");
+    L2_TRY(check_dims(expect));
+    const int fd = open(path, O_RDONLY);
+    if (fd < 0) return l2_fail(L2_ERR_IO, "open %s: %s", path, strerror(errno));
+    struct stat st;
+    if (fstat(fd, &st) != 0) {
+        close(fd);
+        return l2_fail(L2_ERR_IO, "stat %s: %s", path, strerror(errno));
+    }
+    int32_t h[7];
+    if (st.st_size < 28 || pread(fd, h, 28, 0) != 28) {
+        close(fd);
+        return l2_fail(L2_ERR_FORMAT, "%s: shorter than the 28-byte header", path);
+    }
+    // Config::load + check_static (src/constants.rs:94-119)
+    l2_config cfg = {h[0], h[1], h[2], h[3], h[4], h[5] < 0 ? -h[5] : h[5], h[6], h[5] > 0};
+    if (cfg.dim != expect->dim || cfg.hidden_dim != expect->hidden_dim || cfg.n_layers != expect->n_layers ||
+        cfg.n_heads != expect->n_heads || cfg.vocab_size != expect->vocab_size) {
+        close(fd);
+        return l2_fail(L2_ERR_FORMAT,
+                       "%s: header (dim %d, hidden %d, layers %d, heads %d, vocab %d) does not match the "
+                       "expected (%d, %d, %d, %d, %d)",
+                       path, cfg.dim, cfg.hidden_dim, cfg.n_layers, cfg.n_heads, cfg.vocab_size, expect->dim,
+                       expect->hidden_dim, expect->n_layers, expect->n_heads, expect->vocab_size);
+    }
+    const size_t want = l2_weights_bytes(expect);
+    if ((size_t)st.st_size - 28 != want) { // src/lib.rs:97
+        close(fd);
+        return l2_fail(L2_ERR_FORMAT, "%s: %zu bytes after the header, the struct for these dims is %zu", path,
+                       (size_t)st.st_size - 28, want);
+    }
+    // The reference maps from byte 28 (src/lib.rs:95-96); mmap offsets must be
+    // page aligned, so map from 0 and step over the header.
+    void *map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (map == MAP_FAILED) return l2_fail(L2_ERR_IO, "mmap %s: %s", path, strerror(errno));
+    (void)madvise(map, (size_t)st.st_size, MADV_SEQUENTIAL);
+    const int rc = model_build((const char *)map + 28, want, expect, max_seq, out);
+    munmap(map, (size_t)st.st_size);
+    if (rc == L2_OK) (*out)->cfg = cfg;
+    return rc;
+}
+
+extern "C" void l2_model_close(l2_model *m) {
+    if (!m) return;
+    if (m->stream) (void)hipStreamSynchronize(m->stream);
+    void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->x, m->xq, m->xk, m->xv, m->qv,
+                    m->kv, m->vv, m->attg, m->x1, m->x3, m->hb, m->hb2, m->hg, m->fin, m->logits,
+                    m->dtok, m->dpos, m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y};
+    for (void *p : ptrs) dfree(p);
+    if (m->stream) (void)hipStreamDestroy(m->stream);
+    delete m;
+}
+
+extern "C" int l2_model_config(const l2_model *m, l2_config *out) {
+    if (!m || !out) return l2_fail(L2_ERR_ARG, "null argument");
+    *out = m->cfg;
+    return L2_OK;
+}
+
+extern "C" int l2_model_dims(const l2_model *m, l2_dims *out) {
+    if (!m || !out) return l2_fail(L2_ERR_ARG, "null argument");
+    *out = m->d;
+    return L2_OK;
+}
+
+extern "C" int l2_model_max_seq(const l2_model *m) { return m ? m->max_seq : 0; }
+
+extern "C" int l2_prefill_supported(const l2_model *m) { return m ? 1 : 0; }
+
+extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
+    if (!m) return l2_fail(L2_ERR_ARG, "null model");
+    if (mode != L2_PREFILL_FP32) return l2_fail(L2_ERR_ARG, "prefill mode %d is not available", mode);
+    m->prefill_mode = mode;
+    return L2_OK;
+}
+
+static int ensure_batch(l2_model *m, int B) {
+    if (B <= m->cap_B) return L2_OK;
+    L2_HIP(hipStreamSynchronize(m->stream));
+    float **bufs[] = {&m->x, &m->xq, &m->xk, &m->xv, &m->qv, &m->kv, &m->vv, &m->attg,
+                      &m->x1, &m->x3, &m->hb, &m->hb2, &m->hg, &m->fin};
+    for (float **b : bufs) {
+        dfree(*b);
+        *b = nullptr;
+    }
+    dfree(m->dtok);
+    dfree(m->dpos);
+    m->dtok = m->dpos = nullptr;
+    m->cap_B = 0;
+    const size_t dim = m->d.dim, hid = m->d.hidden_dim, kvd = m->kv_dim;
+    L2_TRY(dalloc(&m->x, B * dim));
+    L2_TRY(dalloc(&m->xq, B * dim));
+    L2_TRY(dalloc(&m->xk, B * dim));
+    L2_TRY(dalloc(&m->xv, B * dim));
+    L2_TRY(dalloc(&m->qv, B * dim));
+    L2_TRY(dalloc(&m->kv, B * kvd));
+    L2_TRY(dalloc(&m->vv, B * kvd));
+    L2_TRY(dalloc(&m->attg, B * dim));
+    L2_TRY(dalloc(&m->x1, B * dim));
+    L2_TRY(dalloc(&m->x3, B * dim));
+    L2_TRY(dalloc(&m->hb, B * hid));
+    L2_TRY(dalloc(&m->hb2, B * hid));
+    L2_TRY(dalloc(&m->hg, B * hid));
+    L2_TRY(dalloc(&m->fin, B * dim));
+    L2_TRY(dalloc(&m->dtok, (size_t)B));
+    L2_TRY(dalloc(&m->dpos, (size_t)B));
+    if (!m->logits) L2_TRY(dalloc(&m->logits, (size_t)m->d.vocab_size));
+    m->cap_B = B;
+    return L2_OK;
+}
+
+// ---------------------------------------------------------------------------
+// state
+
+extern "C" int l2_state_new(l2_model *m, l2_state **out) {
+    if (!m || !out) return l2_fail(L2_ERR_ARG, "null argument");
+    l2_state *s = new l2_state();
+    s->m = m;
+    s->elems = (size_t)m->d.n_layers * m->max_seq * m->kv_dim;
+    int rc = dalloc(&s->kcache, s->elems);
+    if (rc == L2_OK) rc = dalloc(&s->vcache, s->elems);
+    if (rc != L2_OK) {
+        l2_state_free(s);
+        return rc;
+    }
+    rc = l2_state_reset(s);
+    if (rc != L2_OK) {
+        l2_state_free(s);
+        return rc;
+    }
+    *out = s;
+    return L2_OK;
+}
+
+extern "C" void l2_state_free(l2_state *s) {
+    if (!s) return;
+    if (s->m && s->m->stream) (void)hipStreamSynchronize(s->m->stream);
+    dfree(s->kcache);
+    dfree(s->vcache);
+    delete s;
+}
+
+extern "C" int l2_state_reset(l2_state *s) {
+    if (!s) return l2_fail(L2_ERR_ARG, "null state");
+    L2_HIP(hipMemsetAsync(s->kcache, 0, s->elems * 4, s->m->stream));
+    L2_HIP(hipMemsetAsync(s->vcache, 0, s->elems * 4, s->m->stream));
+    L2_HIP(hipStreamSynchronize(s->m->stream));
+    return L2_OK;
+}
+
+extern "C" int l2_state_read_kv(l2_state *s, int layer, int pos0, int npos, float *k_host, float *v_host) {
+    if (!s || !k_host || !v_host) return l2_fail(L2_ERR_ARG, "null argument");
+    const l2_model *m = s->m;
+    if (layer < 0 || layer >= m->d.n_layers || pos0 < 0 || npos < 0 || pos0 + npos > m->max_seq)
+        return l2_fail(L2_ERR_RANGE, "read_kv: layer %d, positions [%d,%d)", layer, pos0, pos0 + npos);
+    const size_t off = ((size_t)layer * m->max_seq + pos0) * m->kv_dim;
+    L2_HIP(hipStreamSynchronize(m->stream));
+    L2_HIP(hipMemcpy(k_host, s->kcache + off, (size_t)npos * m->kv_dim * 4, hipMemcpyDeviceToHost));
+    L2_HIP(hipMemcpy(v_host, s->vcache + off, (size_t)npos * m->kv_dim * 4, hipMemcpyDeviceToHost));
+    return L2_OK;
+}
+
+extern "C" int l2_state_fill_synthetic(l2_state *s, int pos0, int npos, uint64_t seed) {
+    if (!s) return l2_fail(L2_ERR_ARG, "null state");
+    const l2_model *m = s->m;
+    if (pos0 < 0 || npos < 0 || pos0 + npos > m->max_seq)
+        return l2_fail(L2_ERR_RANGE, "fill: positions [%d,%d)", pos0, pos0 + npos);
+    for (int l = 0; l < m->d.n_layers; l++) {
+        const size_t off = ((size_t)l * m->max_seq + pos0) * m->kv_dim;
+        const size_t n = (size_t)npos * m->kv_dim;
+        L2_TRY(fill_pattern_launch(s->kcache + off, n, seed * 2654435761ull + 2 * l, m->stream));
+        L2_TRY(fill_pattern_launch(s->vcache + off, n, seed * 2654435761ull + 2 * l + 1, m->stream));
+    }
+    L2_HIP(hipStreamSynchronize(m->stream));
+    return L2_OK;
+}
+
+// ---------------------------------------------------------------------------
+// operators
+
+static Q4Mat mat_of(const DevQLinear &q, const float *x, float *y, int y_stride, const float *res,
+                    const int32_t *scatter) {
+    Q4Mat M{};
+    M.qweight = q.qweight;
+    M.qzeros = q.qzeros;
+    M.scales = q.scales;
+    M.x = x;
+    M.y = y;
+    M.res = res;
+    M.scatter = scatter;
+    M.out = q.out;
+    M.y_stride = y_stride;
+    return M;
+}
+
+static int q4_one(const DevQLinear &q, const float *xg, float *y, const float *res, const int32_t *scatter,
+                  int B, hipStream_t st) {
+    Q4Launch L{};
+    L.m[0] = mat_of(q, xg, y, q.out, res, scatter);
+    L.n_mats = 1;
+    L.in = q.in;
+    L.groups = q.groups;
+    L.group_size = q.group_size;
+    L.epi = res ? Q4_EPI_RESIDUAL : Q4_EPI_STORE;
+    L.batch = B;
+    return q4_matvec_launch(L, st);
+}
+
+static int check_qlinear_shape(int in, int out, int g) {
+    if (g != 32 && g != 64 && g != 128) return l2_fail(L2_ERR_ARG, "group size %d (32, 64 or 128)", g);
+    if (in <= 0 || out <= 0 || in % 32 || in % g || out % 8)
+        return l2_fail(L2_ERR_ARG, "QLinear %dx%d: in must be a multiple of 32 and of the group size, out of 8", in, out);
+    return L2_OK;
+}
+
+extern "C" int l2_qlinear_create(const int32_t *qweight, const int32_t *qzeros, const float *scales,
+                                 const int32_t *g_index, int in, int out, int group_size, l2_qlinear **ql) {
+    if (!qweight || !qzeros || !scales || !g_index || !ql) return l2_fail(L2_ERR_ARG, "null argument");
+    L2_TRY(check_qlinear_shape(in, out, group_size));
+    L2_TRY(require_device());
+    const int groups = (int)div_up(in, group_size);
+    std::vector<int32_t> inv(in);
+    bool ok = true;
+    invert_perm(g_index, in, inv.data(), &ok);
+    if (!ok) return l2_fail(L2_ERR_FORMAT, "g_index is not a permutation of 0..%d", in - 1);
+    l2_qlinear *q = new l2_qlinear();
+    const size_t sizes[5] = {(size_t)out * (in / 8) * 4, (size_t)(out / 8) * groups * 4, (size_t)out * groups * 4,
+                             (size_t)in * 4, (size_t)in * 4};
+    const void *src[5] = {qweight, qzeros, scales, g_index, inv.data()};
+    for (int i = 0; i < 5; i++) {
+        hipError_t e = hipMalloc(&q->bufs[i], sizes[i]);
+        if (e == hipSuccess) e = hipMemcpy(q->bufs[i], src[i], sizes[i], hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            l2_qlinear_free(q);
+            return l2_fail(L2_ERR_HIP, "upload of QLinear array %d: %s", i, hipGetErrorString(e));
+        }
+    }
+    if (hipStreamCreate(&q->stream) != hipSuccess) {
+        l2_qlinear_free(q);
+        return l2_fail(L2_ERR_HIP, "hipStreamCreate failed");
+    }
+    q->q.qweight = (const uint4 *)q->bufs[0];
+    q->q.qzeros = (const int32_t *)q->bufs[1];
+    q->q.scales = (const float *)q->bufs[2];
+    q->q.g_index = (const int32_t *)q->bufs[3];
+    q->q.inv_index = (const int32_t *)q->bufs[4];
+    q->q.in = in;
+    q->q.out = out;
+    q->q.groups = groups;
+    q->q.group_size = group_size;
+    *ql = q;
+    return L2_OK;
+}
+
+extern "C" void l2_qlinear_free(l2_qlinear *q) {
+    if (!q) return;
+    if (q->stream) (void)hipStreamSynchronize(q->stream);
+    for (void *p : q->bufs) dfree(p);
+    dfree(q->x);
+    dfree(q->xg);
+    dfree(q->y);
+    if (q->stream) (void)hipStreamDestroy(q->stream);
+    delete q;
+}
+
+static int qlinear_scratch(l2_qlinear *q, int B) {
+    if (B <= q->cap_B) return L2_OK;
+    dfree(q->x);
+    dfree(q->xg);
+    dfree(q->y);
+    q->x = q->xg = q->y = nullptr;
+    q->cap_B = 0;
+    L2_TRY(dalloc(&q->x, (size_t)B * q->q.in));
+    L2_TRY(dalloc(&q->xg, (size_t)B * q->q.in));
+    L2_TRY(dalloc(&q->y, (size_t)B * q->q.out));
+    q->cap_B = B;
+    return L2_OK;
+}
+
+// x (host, natural order) -> gather through g_index -> matvec -> y (host)
+static int matvec_host(const DevQLinear &q, float *dx, float *dxg, float *dy, const float *x_host, int B,
+                       float *y_host, hipStream_t st) {
+    L2_HIP(hipMemcpyAsync(dx, x_host, (size_t)B * q.in * 4, hipMemcpyHostToDevice, st));
+    L2_TRY(gather_launch(dxg, dx, q.g_index, q.in, B, st));
+    L2_TRY(q4_one(q, dxg, dy, nullptr, nullptr, B, st));
+    L2_HIP(hipMemcpyAsync(y_host, dy, (size_t)B * q.out * 4, hipMemcpyDeviceToHost, st));
+    L2_HIP(hipStreamSynchronize(st));
+    return L2_OK;
+}
+
+extern "C" int l2_qlinear_matvec(l2_qlinear *q, const float *x_host, int B, float *y_host) {
+    if (!q || !x_host || !y_host) return l2_fail(L2_ERR_ARG, "null argument");
+    if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
+    L2_TRY(qlinear_scratch(q, B));
+    return matvec_host(q->q, q->x, q->xg, q->y, x_host, B, y_host, q->stream);
+}
+
+static int op_scratch(l2_model *m, size_t elems) {
+    if (elems <= m->op_cap) return L2_OK;
+    L2_HIP(hipStreamSynchronize(m->stream));
+    dfree(m->op_x);
+    dfree(m->op_xg);
+    dfree(m->op_y);
+    m->op_x = m->op_xg = m->op_y = nullptr;
+    m->op_cap = 0;
+    L2_TRY(dalloc(&m->op_x, elems));
+    L2_TRY(dalloc(&m->op_xg, elems));
+    L2_TRY(dalloc(&m->op_y, elems));
+    m->op_cap = elems;
+    return L2_OK;
+}
+
+extern "C" int l2_model_qmatvec(l2_model *m, int layer, int proj, const float *x_host, int B, float *y_host) {
+    if (!m || !x_host || !y_host) return l2_fail(L2_ERR_ARG, "null argument");
+    if (proj < 0 || proj > 6 || layer < 0 || layer >= m->d.n_layers)
+        return l2_fail(L2_ERR_RANGE, "projection %d, layer %d", proj, layer);
+    if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
+    const DevQLinear &q = m->q[proj][layer];
+    L2_TRY(op_scratch(m, (size_t)B * std::max(std::max(q.in, q.out), m->d.vocab_size)));
+    return matvec_host(q, m->op_x, m->op_xg, m->op_y, x_host, B, y_host, m->stream);
+}
+
+extern "C" int l2_model_classifier(l2_model *m, const float *x_host, float *y_host) {
+    if (!m || !x_host || !y_host) return l2_fail(L2_ERR_ARG, "null argument");
+    L2_TRY(op_scratch(m, (size_t)std::max(m->d.dim, m->d.vocab_size)));
+    L2_HIP(hipMemcpyAsync(m->op_x, x_host, (size_t)m->d.dim * 4, hipMemcpyHostToDevice, m->stream));
+    L2_TRY(dense_matvec_launch(m->op_y, m->wcls, m->op_x, m->d.dim, m->d.vocab_size, nullptr, m->stream));
+    L2_HIP(hipMemcpyAsync(y_host, m->op_y, (size_t)m->d.vocab_size * 4, hipMemcpyDeviceToHost, m->stream));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    return L2_OK;
+}
+
+// ---------------------------------------------------------------------------
+// transformer<B>
+
+// Enqueue one forward pass for the B tokens / positions already in m->dtok /
+// m->dpos.  max_pos is the largest position among them (sizes the attention
+// scratch).  With want_logits the classifier and the running argmax follow.
+static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits) {
+    const l2_dims &d = m->d;
+    const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
+    hipStream_t st = m->stream;
+    L2_TRY(embed_launch(m->x, m->tok_emb, m->dtok, dim, d.vocab_size, B, st)); // :189-191
+    for (int l = 0; l < L; l++) {
+        const DevQLinear &wq = m->q[L2_WQ][l], &wk = m->q[L2_WK][l], &wv = m->q[L2_WV][l],
+                         &wo = m->q[L2_WO][l], &w1 = m->q[L2_W1][l], &w2 = m->q[L2_W2][l],
+                         &w3 = m->q[L2_W3][l];
+        // attention rmsnorm (:217-219), delivered in the three input orders
+        ScatterTargets t{};
+        t.n = 3;
+        t.inv[0] = wq.inv_index, t.inv[1] = wk.inv_index, t.inv[2] = wv.inv_index;
+        t.out[0] = m->xq, t.out[1] = m->xk, t.out[2] = m->xv;
+        L2_TRY(rmsnorm_scatter_launch(m->x, m->rms_att + (size_t)l * dim, m->rms_eps, dim, B, t, st));
+        {   // q, k, v (:224-226) in one launch
+            Q4Launch Q{};
+            Q.m[0] = mat_of(wq, m->xq, m->qv, dim, nullptr, nullptr);
+            Q.m[1] = mat_of(wk, m->xk, m->kv, kvd, nullptr, nullptr);
+            Q.m[2] = mat_of(wv, m->xv, m->vv, kvd, nullptr, nullptr);
+            Q.n_mats = 3;
+            Q.in = dim;
+            Q.groups = wq.groups;
+            Q.group_size = d.group_size;
+            Q.epi = Q4_EPI_STORE;
+            Q.batch = B;
+            L2_TRY(q4_matvec_launch(Q, st));
+        }
+        float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
+        float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
+        // rope + cache write for all B columns (:228-249), then attention (:250-256)
+        L2_TRY(rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
+                              d.n_kv_heads, m->head_size, B, st));
+        L2_TRY(attention_launch(m->attg, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
+                                m->head_size, max_pos, B, st));
+        // wo and the residual (:260-264)
+        L2_TRY(q4_one(wo, m->attg, m->x, m->x, nullptr, B, st));
+        // ffn rmsnorm (:266), w1 | w3 (:271-272), silu gate (:274-276), w2 + residual (:279-285)
+        ScatterTargets t2{};
+        t2.n = 2;
+        t2.inv[0] = w1.inv_index, t2.inv[1] = w3.inv_index;
+        t2.out[0] = m->x1, t2.out[1] = m->x3;
+        L2_TRY(rmsnorm_scatter_launch(m->x, m->rms_ffn + (size_t)l * dim, m->rms_eps, dim, B, t2, st));
+        {
+            Q4Launch Q{};
+            Q.m[0] = mat_of(w1, m->x1, m->hb, hid, nullptr, nullptr);
+            Q.m[1] = mat_of(w3, m->x3, m->hb2, hid, nullptr, nullptr);
+            Q.n_mats = 2;
+            Q.in = dim;
+            Q.groups = w1.groups;
+            Q.group_size = d.group_size;
+            Q.epi = Q4_EPI_STORE;
+            Q.batch = B;
+            L2_TRY(q4_matvec_launch(Q, st));
+        }
+        L2_TRY(silu_scatter_launch(m->hg, m->hb, m->hb2, w2.inv_index, hid, B, st));
+        L2_TRY(q4_one(w2, m->hg, m->x, m->x, nullptr, B, st));
+    }
+    if (want_logits) { // :288-297, B == 1 only
+        ScatterTargets t{};
+        t.n = 1;
+        t.inv[0] = nullptr;
+        t.out[0] = m->fin;
+        L2_TRY(rmsnorm_scatter_launch(m->x, m->rms_final, m->rms_eps, dim, 1, t, st));
+        L2_TRY(fill_u64_launch(m->amax, 0ull, 1, st));
+        L2_TRY(dense_matvec_launch(m->logits, m->wcls, m->fin, dim, d.vocab_size, m->amax, st));
+    }
+    return L2_OK;
+}
+
+static int check_tokens(const l2_model *m, const int32_t *tokens, const int32_t *pos, int B, int *max_pos) {
+    int mp = 0;
+    for (int b = 0; b < B; b++) {
+        if (tokens[b] < 0 || tokens[b] >= m->d.vocab_size)
+            return l2_fail(L2_ERR_RANGE, "token id %d outside 0..%d", tokens[b], m->d.vocab_size - 1);
+        if (pos[b] < 0 || pos[b] >= m->max_seq)
+            return l2_fail(L2_ERR_RANGE, "position %d outside 0..%d", pos[b], m->max_seq - 1);
+        mp = std::max(mp, pos[b]);
+    }
+    *max_pos = mp;
+    return L2_OK;
+}
+
+extern "C" int l2_forward(l2_model *m, l2_state *s, const int32_t *tokens, const int32_t *pos, int B,
+                          float *logits_host) {
+    if (!m || !s || !tokens || !pos) return l2_fail(L2_ERR_ARG, "null argument");
+    if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
+    if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
+    int max_pos = 0;
+    L2_TRY(check_tokens(m, tokens, pos, B, &max_pos));
+    L2_TRY(ensure_batch(m, B));
+    L2_HIP(hipMemcpyAsync(m->dtok, tokens, (size_t)B * 4, hipMemcpyHostToDevice, m->stream));
+    L2_HIP(hipMemcpyAsync(m->dpos, pos, (size_t)B * 4, hipMemcpyHostToDevice, m->stream));
+    L2_TRY(forward_enqueue(m, s, B, max_pos, B == 1));
+    if (B == 1 && logits_host)
+        L2_HIP(hipMemcpyAsync(logits_host, m->logits, (size_t)m->d.vocab_size * 4, hipMemcpyDeviceToHost, m->stream));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    return L2_OK;
+}
+
+extern "C" int l2_decode_greedy(l2_model *m, l2_state *s, int32_t token, int32_t pos, int32_t *next) {
+    if (!m || !s || !next) return l2_fail(L2_ERR_ARG, "null argument");
+    if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
+    int max_pos = 0;
+    L2_TRY(check_tokens(m, &token, &pos, 1, &max_pos));
+    L2_TRY(ensure_batch(m, 1));
+    L2_HIP(hipMemcpyAsync(m->dtok, &token, 4, hipMemcpyHostToDevice, m->stream));
+    L2_HIP(hipMemcpyAsync(m->dpos, &pos, 4, hipMemcpyHostToDevice, m->stream));
+    L2_TRY(forward_enqueue(m, s, 1, pos, true));
+    unsigned long long key = 0;
+    L2_HIP(hipMemcpyAsync(&key, m->amax, 8, hipMemcpyDeviceToHost, m->stream));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    *next = (int32_t)(key & 0xFFFFFFFFull);
+    return L2_OK;
+}
+
+static int ensure_loop_buffers(l2_model *m, int n_prompt, int n_out) {
+    if (n_prompt > m->cap_prompt) {
+        L2_HIP(hipStreamSynchronize(m->stream));
+        dfree(m->dprompt);
+        m->dprompt = nullptr;
+        m->cap_prompt = 0;
+        L2_TRY(dalloc(&m->dprompt, (size_t)n_prompt));
+        m->cap_prompt = n_prompt;
+    }
+    if (n_out > m->cap_out) {
+        L2_HIP(hipStreamSynchronize(m->stream));
+        dfree(m->dout_ids);
+        m->dout_ids = nullptr;
+        m->cap_out = 0;
+        L2_TRY(dalloc(&m->dout_ids, (size_t)n_out));
+        m->cap_out = n_out;
+    }
+    return L2_OK;
+}
+
+// The B=1 loop body with everything on the device: forward from m->dtok at
+// m->dpos (== pos, which the host tracks only to size the attention scratch),
+// then next = prompt[pos] if still inside the prompt else argmax
+// (src/inference.rs:146-162), stored to out_ids[pos - pos0], fed back as the
+// token, and the device position advanced.
+static int loop_step(l2_model *m, l2_state *s, int pos, int n_prompt, int pos0) {
+    L2_TRY(forward_enqueue(m, s, 1, pos, true));
+    L2_TRY(next_token_launch(m->amax, m->dprompt, n_prompt, m->dpos, m->dout_ids, pos0, m->dtok, m->stream));
+    return L2_OK;
+}
+
+extern "C" int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *prompt, int n_prompt, int steps,
+                                  int use_prefill, int32_t *out_ids, int *n_out, double *ms) {
+    if (!m || !s || !out_ids || !n_out || (n_prompt > 0 && !prompt)) return l2_fail(L2_ERR_ARG, "null argument");
+    if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
+    if (n_prompt < 0 || steps < 0) return l2_fail(L2_ERR_ARG, "negative count");
+    if (steps > m->max_seq) return l2_fail(L2_ERR_RANGE, "steps %d exceeds the cache length %d", steps, m->max_seq);
+    for (int i = 0; i < n_prompt; i++)
+        if (prompt[i] < 0 || prompt[i] >= m->d.vocab_size)
+            return l2_fail(L2_ERR_RANGE, "prompt token %d outside 0..%d", prompt[i], m->d.vocab_size - 1);
+    L2_TRY(l2_state_reset(s)); // RunState::new per call (:59)
+    L2_TRY(ensure_batch(m, use_prefill ? 64 : 1));
+    L2_TRY(ensure_loop_buffers(m, std::max(n_prompt, 1), std::max(steps, 1)));
+    if (n_prompt > 0)
+        L2_HIP(hipMemcpyAsync(m->dprompt, prompt, (size_t)n_prompt * 4, hipMemcpyHostToDevice, m->stream));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    const auto t0 = std::chrono::steady_clock::now(); // :72
+    int pos = 0;
+    if (use_prefill) { // :78-127
+        static const int ladder[6] = {64, 32, 16, 8, 4, 2};
+        std::vector<int32_t> toks(64), poss(64);
+        for (int A : ladder) {
+            while (pos + A < n_prompt) { // :24
+                for (int i = 0; i < A; i++) {
+                    toks[i] = pos == 0 ? 1 : prompt[pos - 1]; // START, :29-33
+                    poss[i] = pos;
+                    pos++;
+                }
+                L2_HIP(hipMemcpyAsync(m->dtok, toks.data(), (size_t)A * 4, hipMemcpyHostToDevice, m->stream));
+                L2_HIP(hipMemcpyAsync(m->dpos, poss.data(), (size_t)A * 4, hipMemcpyHostToDevice, m->stream));
+                L2_TRY(forward_enqueue(m, s, A, pos - 1, false));
+                L2_HIP(hipStreamSynchronize(m->stream)); // toks/poss are reused
+            }
+        }
+    }
+    const int32_t first = pos == 0 ? 1 : prompt[pos - 1]; // :128-132
+    L2_TRY(set_i32_launch(m->dtok, first, m->dpos, pos, m->stream));
+    const int pos0 = pos;
+    int n = 0;
+    while (pos < steps) { // :141
+        L2_TRY(loop_step(m, s, pos, n_prompt, pos0));
+        n++;
+        pos++;
+    }
+    L2_HIP(hipStreamSynchronize(m->stream));
+    const auto t1 = std::chrono::steady_clock::now(); // :192
+    if (n > 0) L2_HIP(hipMemcpy(out_ids, m->dout_ids, (size_t)n * 4, hipMemcpyDeviceToHost));
+    *n_out = n;
+    if (ms) *ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    return L2_OK;
+}
+
+// ---------------------------------------------------------------------------
+// measurement hooks
+
+extern "C" int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_total) {
+    if (!qs || n < 1 || iters < 1 || !ms_total) return l2_fail(L2_ERR_ARG, "bad argument");
+    hipStream_t st = qs[0]->stream;
+    for (int i = 0; i < n; i++) {
+        if (!qs[i]) return l2_fail(L2_ERR_ARG, "null qlinear %d", i);
+        L2_TRY(qlinear_scratch(qs[i], 1));
+        L2_TRY(fill_pattern_launch(qs[i]->xg, (size_t)qs[i]->q.in, 17 + i, st));
+    }
+    hipEvent_t e0, e1;
+    L2_HIP(hipEventCreate(&e0));
+    L2_HIP(hipEventCreate(&e1));
+    for (int i = 0; i < n; i++) L2_TRY(q4_one(qs[i]->q, qs[i]->xg, qs[i]->y, nullptr, nullptr, 1, st)); // warm-up
+    L2_HIP(hipStreamSynchronize(st));
+    L2_HIP(hipEventRecord(e0, st));
+    for (int it = 0; it < iters; it++) {
+        l2_qlinear *q = qs[it % n];
+        L2_TRY(q4_one(q->q, q->xg, q->y, nullptr, nullptr, 1, st));
+    }
+    L2_HIP(hipEventRecord(e1, st));
+    L2_HIP(hipEventSynchronize(e1));
+    L2_HIP(hipEventElapsedTime(ms_total, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return L2_OK;
+}
+
+extern "C" int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
+                               int32_t *out_ids, float *ms_total) {
+    if (!m || !s || !ms_total || n_tokens < 1) return l2_fail(L2_ERR_ARG, "bad argument");
+    if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
+    if (pos < 0 || pos + n_tokens > m->max_seq) return l2_fail(L2_ERR_RANGE, "positions [%d,%d) exceed the cache", pos, pos + n_tokens);
+    if (token < 0 || token >= m->d.vocab_size) return l2_fail(L2_ERR_RANGE, "token %d", token);
+    L2_TRY(ensure_batch(m, 1));
+    L2_TRY(ensure_loop_buffers(m, 1, n_tokens));
+    L2_TRY(set_i32_launch(m->dtok, token, m->dpos, pos, m->stream));
+    hipEvent_t e0, e1;
+    L2_HIP(hipEventCreate(&e0));
+    L2_HIP(hipEventCreate(&e1));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    L2_HIP(hipEventRecord(e0, m->stream));
+    for (int i = 0; i < n_tokens; i++) L2_TRY(loop_step(m, s, pos + i, 0, pos));
+    L2_HIP(hipEventRecord(e1, m->stream));
+    L2_HIP(hipEventSynchronize(e1));
+    L2_HIP(hipEventElapsedTime(ms_total, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (out_ids) L2_HIP(hipMemcpy(out_ids, m->dout_ids, (size_t)n_tokens * 4, hipMemcpyDeviceToHost));
+    return L2_OK;
+}
+
+extern "C" int l2_copy_bench(size_t nbytes, int iters, float *ms_total) {
+    if (!ms_total || nbytes < 16 || iters < 1) return l2_fail(L2_ERR_ARG, "bad argument");
+    L2_TRY(require_device());
+    char *a = nullptr, *b = nullptr;
+    L2_TRY(dalloc(&a, nbytes));
+    if (dalloc(&b, nbytes) != L2_OK) {
+        dfree(a);
+        return L2_ERR_HIP;
+    }
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    (void)hipMemcpyAsync(b, a, nbytes, hipMemcpyDeviceToDevice, nullptr);
+    (void)hipDeviceSynchronize();
+    (void)hipEventRecord(e0, nullptr);
+    for (int i = 0; i < iters; i++) (void)hipMemcpyAsync(b, a, nbytes, hipMemcpyDeviceToDevice, nullptr);
+    (void)hipEventRecord(e1, nullptr);
+    hipError_t e = hipEventSynchronize(e1);
+    if (e == hipSuccess) e = hipEventElapsedTime(ms_total, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    dfree(a);
+    dfree(b);
+    if (e != hipSuccess) return l2_fail(L2_ERR_HIP, "copy bench: %s", hipGetErrorString(e));
+    return L2_OK;
+}

@@ -1,0 +1,400 @@
+// The per-token kernels around the q4 matvec: embedding gather, RMSNorm, RoPE +
+// KV-cache write, GQA attention, SiLU gate, the fp32 classifier with a fused
+// argmax, and the greedy loop's token hand-over.  gfx950, wave64.
+//
+// This file is compiled with -ffp-contract=off: wherever the reference rounds
+// a product before adding (Rust never fuses), so does this code; FMAs appear
+// only where written as fmaf().
+//
+// "scatter" arguments are inverse act-order permutations: a producer writes
+// element i of its result to slot inv[i] of the buffer the next QLinear reads,
+// which is that layer's x[g_index[j]] gather (src/gptq.rs:110-114) done once
+// at the source instead of once per consumer block.
+#include "l2_internal.h"
+
+namespace {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_xchg(float v) {
+    int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+    return __builtin_bit_cast(float, r);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_xchg<0xB1>(v);
+    v += dpp_xchg<0x4E>(v);
+    v += dpp_xchg<0x141>(v);
+    v += dpp_xchg<0x140>(v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_xchg<0xB1>(v));
+    v = fmaxf(v, dpp_xchg<0x4E>(v));
+    v = fmaxf(v, dpp_xchg<0x141>(v));
+    v = fmaxf(v, dpp_xchg<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+
+// Block-wide sum / max for blocks of up to 1024 threads; `red` holds 16 floats.
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (int i = 0; i < nw; i++) s += red[i];
+    return s;
+}
+
+__device__ __forceinline__ float block_max(float v, float *red) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float s = red[0];
+    for (int i = 1; i < nw; i++) s = fmaxf(s, red[i]);
+    return s;
+}
+
+// x[b] = token_embedding_table[token[b]]  (src/models.rs:189-191)
+__global__ void embed_kernel(float *x, const float *emb, const int32_t *tokens, int dim) {
+    const int b = blockIdx.x;
+    const float4 *src = reinterpret_cast<const float4 *>(emb + (size_t)tokens[b] * dim);
+    float4 *dst = reinterpret_cast<float4 *>(x + (size_t)b * dim);
+    for (int i = threadIdx.x; i < dim / 4; i += blockDim.x) dst[i] = src[i];
+}
+
+// rmsnorm (src/models.rs:53-66): o[j] = (w[j] * ss) * x[j], ss = 1/sqrt(mean(x^2) + eps),
+// written through up to three inverse permutations.
+__global__ __launch_bounds__(1024) void rmsnorm_scatter_kernel(const float *x, const float *w, float eps,
+                                                                int dim, ScatterTargets t) {
+    __shared__ float red[16];
+    const int b = blockIdx.x;
+    const float *xb = x + (size_t)b * dim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) ss = fmaf(xb[i], xb[i], ss);
+    ss = block_sum(ss, red);
+    ss /= (float)dim;
+    ss += eps;
+    ss = 1.0f / sqrtf(ss);
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        const float v = w[i] * ss * xb[i];
+        for (int c = 0; c < t.n; c++) {
+            const int dst = t.inv[c] ? t.inv[c][i] : i;
+            t.out[c][(size_t)b * dim + dst] = v;
+        }
+    }
+}
+
+// out[b][j] = x[b][g_index[j]]  (src/gptq.rs:110-114), for callers that hand the
+// operator an input in natural order.
+__global__ void gather_kernel(float *out, const float *x, const int32_t *g_index, int n) {
+    const int b = blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < n) out[(size_t)b * n + j] = x[(size_t)b * n + g_index[j]];
+}
+
+// rope (src/models.rs:100-129) on q in place and on k while it is copied into
+// the cache, v copied beside it (:236-249).  The second half of a head uses the
+// first half's ROTATED value, as the reference's in-place loop does.
+// One block per (batch column); thread -> (head, i < half).
+__global__ void rope_kv_kernel(float *q, const float *k, const float *v, const int32_t *pos,
+                               const float *cos_t, const float *sin_t, float *kcache, float *vcache,
+                               int n_heads, int n_kv_heads, int head_size) {
+    const int b = blockIdx.x;
+    const int half = head_size >> 1;
+    const int dim = n_heads * head_size, kv_dim = n_kv_heads * head_size;
+    const int p = pos[b];
+    const float *ct = cos_t + (size_t)p * half;
+    const float *st = sin_t + (size_t)p * half;
+    float *qb = q + (size_t)b * dim;
+    const float *kb = k + (size_t)b * kv_dim;
+    const float *vb = v + (size_t)b * kv_dim;
+    float *kc = kcache + (size_t)p * kv_dim;
+    float *vc = vcache + (size_t)p * kv_dim;
+    for (int idx = threadIdx.x; idx < n_heads * half; idx += blockDim.x) {
+        const int h = idx / half, i = idx - h * half;
+        const float c = ct[i], s = st[i];
+        float *qh = qb + h * head_size;
+        const float a = qh[i], bb = qh[i + half];
+        const float first = a * c - bb * s;
+        const float second = bb * c + first * s;
+        qh[i] = first;
+        qh[i + half] = second;
+        if (h < n_kv_heads) {
+            const float *kh = kb + h * head_size;
+            const float ka = kh[i], kb2 = kh[i + half];
+            const float kf = ka * c - kb2 * s;
+            const float ks = kb2 * c + kf * s;
+            kc[h * head_size + i] = kf;
+            kc[h * head_size + i + half] = ks;
+        }
+    }
+    for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) vc[i] = vb[i];
+}
+
+// multihead_attention (src/models.rs:131-176) for one (head, batch column):
+// scores over t = 0..=pos against the kv head h / attn_groups, softmax with
+// max subtraction and division by the sum (:68-81), then the weighted sum of V.
+// Dynamic LDS: att[pos+1].  head_size must be 128.
+__global__ __launch_bounds__(256) void attention_kernel(float *out, const float *q, const float *kcache,
+                                                         const float *vcache, const int32_t *pos,
+                                                         const int32_t *scatter, int n_heads,
+                                                         int n_kv_heads) {
+    constexpr int HS = 128;
+    extern __shared__ float att[];
+    __shared__ float qs[HS];
+    __shared__ float red[16];
+    __shared__ float part[HS];
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
+    const int p = pos[b];
+    const int kvh = h / (n_heads / n_kv_heads);
+    const int tid = threadIdx.x;
+    if (tid < HS) qs[tid] = q[(size_t)b * dim + h * HS + tid];
+    __syncthreads();
+    const float inv_div = sqrtf((float)HS);
+    // scores: 4 lanes per timestep, 32 dims each
+    const int sub = tid & 3;
+    for (int t = tid >> 2; t <= p; t += 64) {
+        const float4 *kr = reinterpret_cast<const float4 *>(kcache + (size_t)t * kv_dim + kvh * HS + sub * 32);
+        const float4 *qr = reinterpret_cast<const float4 *>(qs + sub * 32);
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float4 kk = kr[i], qq = qr[i];
+            s = fmaf(qq.x, kk.x, s);
+            s = fmaf(qq.y, kk.y, s);
+            s = fmaf(qq.z, kk.z, s);
+            s = fmaf(qq.w, kk.w, s);
+        }
+        s += dpp_xchg<0xB1>(s);
+        s += dpp_xchg<0x4E>(s);
+        if (sub == 0) att[t] = s / inv_div;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int t = tid; t <= p; t += 256) m = fmaxf(m, att[t]);
+    m = block_max(m, red);
+    float sum = 0.f;
+    for (int t = tid; t <= p; t += 256) {
+        const float e = expf(att[t] - m);
+        att[t] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, red);
+    for (int t = tid; t <= p; t += 256) att[t] = att[t] / sum;
+    __syncthreads();
+    // weighted values: thread -> (dim d, parity of t)
+    const int d = tid & (HS - 1), par = tid >> 7;
+    float acc = 0.f;
+    for (int t = par; t <= p; t += 2)
+        acc = fmaf(att[t], vcache[(size_t)t * kv_dim + kvh * HS + d], acc);
+    if (par == 1) part[d] = acc;
+    __syncthreads();
+    if (par == 0) {
+        acc += part[d];
+        const int i = h * HS + d;
+        const int dst = scatter ? scatter[i] : i;
+        out[(size_t)b * dim + dst] = acc;
+    }
+}
+
+// silu gate (src/models.rs:92-98): s = s * (1 / (1 + exp(-s))), then s = s * s2.
+__global__ void silu_scatter_kernel(float *out, const float *a, const float *b2, const int32_t *scatter,
+                                    int n) {
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = a[(size_t)b * n + i];
+    s = s * (1.0f / (1.0f + expf(-s)));
+    s = s * b2[(size_t)b * n + i];
+    const int dst = scatter ? scatter[i] : i;
+    out[(size_t)b * n + dst] = s;
+}
+
+// Order-preserving key for (value, index): larger value wins, equal values ->
+// larger index wins, which is util::argmax's last-index rule (src/util.rs:39-46).
+__device__ __forceinline__ unsigned long long amax_key(float v, int idx) {
+    if (v == 0.0f) v = 0.0f; // -0.0 and +0.0 compare equal in the reference
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return ((unsigned long long)u << 32) | (uint32_t)idx;
+}
+
+// Linear::matvec (src/model.rs:22-31) for the classifier: one wave per row,
+// two rows in flight, x staged in LDS.  Optionally folds each logit into a
+// 64-bit (value,index) maximum.
+__global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float *w, const float *x, int in,
+                                                            int out, unsigned long long *amax) {
+    extern __shared__ float xs[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < in / 4; i += 256)
+        reinterpret_cast<float4 *>(xs)[i] = reinterpret_cast<const float4 *>(x)[i];
+    __syncthreads();
+    const int n4 = in / 4;
+    const int waves_total = gridDim.x * 4;
+    for (int o = (blockIdx.x * 4 + wave) * 2; o < out; o += waves_total * 2) {
+        const int o1 = min(o + 1, out - 1);
+        const float4 *r0 = reinterpret_cast<const float4 *>(w + (size_t)o * in);
+        const float4 *r1 = reinterpret_cast<const float4 *>(w + (size_t)o1 * in);
+        float a0 = 0.f, a1 = 0.f;
+        for (int j = lane; j < n4; j += 64) {
+            const float4 xv = reinterpret_cast<const float4 *>(xs)[j];
+            const float4 w0 = r0[j], w1 = r1[j];
+            a0 = fmaf(w0.x, xv.x, a0);
+            a0 = fmaf(w0.y, xv.y, a0);
+            a0 = fmaf(w0.z, xv.z, a0);
+            a0 = fmaf(w0.w, xv.w, a0);
+            a1 = fmaf(w1.x, xv.x, a1);
+            a1 = fmaf(w1.y, xv.y, a1);
+            a1 = fmaf(w1.z, xv.z, a1);
+            a1 = fmaf(w1.w, xv.w, a1);
+        }
+        a0 = wave_sum(a0);
+        a1 = wave_sum(a1);
+        if (lane == 0) {
+            y[o] = a0;
+            unsigned long long key = amax_key(a0, o);
+            if (o + 1 < out) {
+                y[o + 1] = a1;
+                const unsigned long long k1 = amax_key(a1, o + 1);
+                key = k1 > key ? k1 : key;
+            }
+            if (amax) atomicMax(amax, key);
+        }
+    }
+}
+
+__global__ void fill_u64_kernel(unsigned long long *p, unsigned long long v, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// Greedy hand-over (src/inference.rs:154-162, 185-189): next is the forced
+// prompt token while pos < n_prompt, else the argmax; it is recorded, fed back
+// as the next input token, and the position advances -- all without the host.
+__global__ void next_token_kernel(const unsigned long long *amax, const int32_t *prompt, int n_prompt,
+                                  int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const int pos = dpos[0];
+        const int32_t next = pos < n_prompt ? prompt[pos] : (int32_t)(amax[0] & 0xFFFFFFFFull);
+        if (out_ids) out_ids[pos - pos0] = next;
+        tok[0] = next;
+        dpos[0] = pos + 1;
+    }
+}
+
+__global__ void set_i32_kernel(int32_t *p, int32_t a, int32_t *q, int32_t b) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        p[0] = a;
+        if (q) q[0] = b;
+    }
+}
+
+__global__ void fill_pattern_kernel(float *p, size_t n, uint64_t seed) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (i + 1);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    p[i] = (float)((double)(z >> 11) * (1.0 / 9007199254740992.0) * 2.0 - 1.0);
+}
+
+} // namespace
+
+int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int vocab, int B,
+                 hipStream_t st) {
+    (void)vocab;
+    if (dim % 4) return l2_fail(L2_ERR_ARG, "embed: dim=%d not a multiple of 4", dim);
+    hipLaunchKernelGGL(embed_kernel, dim3(B), dim3(256), 0, st, x, emb, tokens, dim);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int rmsnorm_scatter_launch(const float *x, const float *w, float eps, int dim, int B,
+                           const ScatterTargets &t, hipStream_t st) {
+    if (t.n < 1 || t.n > 3) return l2_fail(L2_ERR_ARG, "rmsnorm: %d targets", t.n);
+    hipLaunchKernelGGL(rmsnorm_scatter_kernel, dim3(B), dim3(1024), 0, st, x, w, eps, dim, t);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int gather_launch(float *out, const float *x, const int32_t *g_index, int n, int B, hipStream_t st) {
+    hipLaunchKernelGGL(gather_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, x, g_index, n);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int rope_kv_launch(float *q, const float *k, const float *v, const int32_t *pos, const float *cos_t,
+                   const float *sin_t, float *kcache_l, float *vcache_l, int n_heads, int n_kv_heads,
+                   int head_size, int B, hipStream_t st) {
+    hipLaunchKernelGGL(rope_kv_kernel, dim3(B), dim3(1024), 0, st, q, k, v, pos, cos_t, sin_t, kcache_l,
+                       vcache_l, n_heads, n_kv_heads, head_size);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int attention_launch(float *out, const float *q, const float *kcache_l, const float *vcache_l,
+                     const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
+                     int head_size, int max_pos, int B, hipStream_t st) {
+    if (head_size != 128) return l2_fail(L2_ERR_ARG, "attention: head_size=%d (128 only)", head_size);
+    const size_t lds = (size_t)(max_pos + 1) * sizeof(float);
+    if (lds > 60 * 1024) return l2_fail(L2_ERR_RANGE, "attention: position %d too deep for this kernel", max_pos);
+    hipLaunchKernelGGL(attention_kernel, dim3(n_heads, B), dim3(256), lds, st, out, q, kcache_l, vcache_l,
+                       pos, scatter, n_heads, n_kv_heads);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int silu_scatter_launch(float *out, const float *a, const float *b, const int32_t *scatter, int n,
+                        int B, hipStream_t st) {
+    hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, a, b, scatter, n);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int dense_matvec_launch(float *y, const float *w, const float *x, int in, int out,
+                        unsigned long long *amax_key, hipStream_t st) {
+    if (in % 4 || in * 4 > 64 * 1024) return l2_fail(L2_ERR_ARG, "dense matvec: in=%d", in);
+    int blocks = (out + 7) / 8;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(dense_matvec_kernel, dim3(blocks), dim3(256), (size_t)in * 4, st, y, w, x, in, out,
+                       amax_key);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int fill_u64_launch(unsigned long long *p, unsigned long long v, int n, hipStream_t st) {
+    hipLaunchKernelGGL(fill_u64_kernel, dim3((n + 255) / 256), dim3(256), 0, st, p, v, n);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,
+                      int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok, hipStream_t st) {
+    hipLaunchKernelGGL(next_token_kernel, dim3(1), dim3(64), 0, st, amax_key, prompt, n_prompt, dpos,
+                       out_ids, pos0, tok);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int set_i32_launch(int32_t *p, int32_t a, int32_t *q, int32_t b, hipStream_t st) {
+    hipLaunchKernelGGL(set_i32_kernel, dim3(1), dim3(64), 0, st, p, a, q, b);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int fill_pattern_launch(float *p, size_t n, uint64_t seed, hipStream_t st) {
+    hipLaunchKernelGGL(fill_pattern_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, n, seed);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}

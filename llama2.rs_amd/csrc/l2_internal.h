@@ -1,0 +1,110 @@
+// Internal declarations shared by the host code and the kernel launchers.
+// Not part of the C ABI (that is include/llama2_hip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "../../include/llama2_hip.h"
+
+// ---- error plumbing -------------------------------------------------------
+int l2_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define L2_HIP(call)                                                                     \
+    do {                                                                                 \
+        hipError_t e_ = (call);                                                          \
+        if (e_ != hipSuccess)                                                            \
+            return l2_fail(L2_ERR_HIP, "%s: %s (%s:%d)", #call, hipGetErrorString(e_),   \
+                           __FILE__, __LINE__);                                          \
+    } while (0)
+
+#define L2_TRY(call)            \
+    do {                        \
+        int rc_ = (call);       \
+        if (rc_ != L2_OK) return rc_; \
+    } while (0)
+
+// ---- device views ---------------------------------------------------------
+
+// One QLinear resident in device memory, `.bin` layout (src/gptq.rs:68-84),
+// plus the inverse of g_index so that a producer can write its output straight
+// into the order this layer reads it in.
+struct DevQLinear {
+    const uint4 *qweight = nullptr;   // [out][in/32] chunks of 32 nibbles
+    const int32_t *qzeros = nullptr;  // [out/8][groups]
+    const float *scales = nullptr;    // [out][groups]
+    const int32_t *g_index = nullptr; // [in]
+    const int32_t *inv_index = nullptr; // [in], inv_index[g_index[j]] = j
+    int in = 0, out = 0, groups = 0, group_size = 0;
+};
+
+// ---- q4 matvec launch description ------------------------------------------
+
+enum { Q4_EPI_STORE = 0, Q4_EPI_RESIDUAL = 1 };
+
+struct Q4Mat {
+    const uint4 *qweight;
+    const int32_t *qzeros;
+    const float *scales;
+    const float *x;         // input already in this layer's g_index order: [B][in]
+    float *y;               // [B][y_stride]
+    const float *res;       // Q4_EPI_RESIDUAL: y = res + W x   (may alias y)
+    const int32_t *scatter; // optional: write y[b][scatter[o]] instead of y[b][o]
+    int out;
+    int y_stride;
+    int row_blocks;         // blocks of grid.x that belong to this matrix
+};
+
+struct Q4Launch {
+    Q4Mat m[3];
+    int n_mats;
+    int in;      // shared by all matrices of one launch
+    int groups;
+    int group_size;
+    int epi;
+    int batch;
+};
+
+// Launch the B=1-per-column fp32 dequant matvec for up to 3 matrices that share
+// `in` (e.g. wq|wk|wv or w1|w3).  Fills row_blocks itself.
+int q4_matvec_launch(Q4Launch &L, hipStream_t stream);
+
+// ---- the other per-token kernels -------------------------------------------
+
+struct ScatterTargets {
+    const int32_t *inv[3];
+    float *out[3];
+    int n;
+};
+
+int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int vocab, int B,
+                 hipStream_t st);
+// out_c[b][inv_c[i]] = (w[i] * ss_b) * x[b][i]; inv == nullptr writes in place order.
+int rmsnorm_scatter_launch(const float *x, const float *w, float eps, int dim, int B,
+                           const ScatterTargets &t, hipStream_t st);
+int gather_launch(float *out, const float *x, const int32_t *g_index, int n, int B, hipStream_t st);
+int rope_kv_launch(float *q, const float *k, const float *v, const int32_t *pos, const float *cos_t,
+                   const float *sin_t, float *kcache_l, float *vcache_l, int n_heads, int n_kv_heads,
+                   int head_size, int B, hipStream_t st);
+// out[b][scatter[i]] (or out[b][i]) = attention for query b at position pos[b].
+int attention_launch(float *out, const float *q, const float *kcache_l, const float *vcache_l,
+                     const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
+                     int head_size, int max_pos, int B, hipStream_t st);
+int silu_scatter_launch(float *out, const float *a, const float *b, const int32_t *scatter, int n,
+                        int B, hipStream_t st);
+// y[o] = sum_i w[o][i] x[i]; if amax_key != nullptr also folds (value,index) into it.
+int dense_matvec_launch(float *y, const float *w, const float *x, int in, int out,
+                        unsigned long long *amax_key, hipStream_t st);
+int fill_u64_launch(unsigned long long *p, unsigned long long v, int n, hipStream_t st);
+// pos = dpos[0]; next = pos < n_prompt ? prompt[pos] : index(amax_key);
+// out_ids[pos - pos0] = next; tok[0] = next; dpos[0] = pos + 1.
+int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,
+                      int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok, hipStream_t st);
+// p[0] = a; if (q) q[0] = b.  Scalars travel as kernel arguments, never as
+// asynchronous copies from the caller's stack.
+int set_i32_launch(int32_t *p, int32_t a, int32_t *q, int32_t b, hipStream_t st);
+int fill_pattern_launch(float *p, size_t n, uint64_t seed, hipStream_t st);
