@@ -187,12 +187,20 @@ int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *prompt, int n_pr
  * the launch stream.  *ms_total is the elapsed time of all iters launches. */
 int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_total);
 
-/* Decode `n_tokens` greedy steps from (token,pos) with HIP events around the
- * whole run; out_ids may be NULL.  *ms_total excludes nothing but the final
- * copy of ids.  If kernel_ms is non-NULL it receives per-kernel-class event
- * time (ms, summed over the run) in the order of l2_kernel_class_name(). */
+/* Decode `n_tokens` greedy steps from (token,pos), the argmax fed back on the
+ * device, with HIP events around the whole run on the launch stream; out_ids
+ * may be NULL. */
 int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
                     int32_t *out_ids, float *ms_total);
+
+/* The same loop with a pair of HIP events around every kernel launch (so it
+ * runs slower than l2_decode_bench): per kernel class, the summed event time
+ * in ms and the number of launches.  Arrays hold l2_kernel_class_count()
+ * entries, named by l2_kernel_class_name(). */
+int l2_kernel_class_count(void);
+const char *l2_kernel_class_name(int cls);
+int l2_decode_profile(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
+                      float *ms_by_class, int32_t *launches_by_class);
 
 /* Plain device-to-device copy of nbytes, iters times: the box's achievable
  * copy bandwidth (bytes moved = 2*nbytes per iteration). */

@@ -272,11 +272,14 @@ struct l2_model {
     int32_t *dinv = nullptr;      // all inverse permutations
     float *rope_cos = nullptr, *rope_sin = nullptr; // [max_seq][head_size/2]
 
-    // forward scratch, sized for cap_B batch columns
+    float *dwn = nullptr;         // norm weights in consumer order: [L][5][dim] (q, k, v, w1, w3)
+    float *attn_part = nullptr;   // split-KV workspace [n_heads][kMaxSplits][130]
+
+    // forward scratch, sized for cap_B batch columns.  xq/xk/xv and x1/x3 hold
+    // the raw residual stream in the input order of the named projection.
     int cap_B = 0;
     float *x = nullptr, *xq = nullptr, *xk = nullptr, *xv = nullptr, *qv = nullptr, *kv = nullptr,
-          *vv = nullptr, *attg = nullptr, *x1 = nullptr, *x3 = nullptr, *hb = nullptr, *hb2 = nullptr,
-          *hg = nullptr, *fin = nullptr, *logits = nullptr;
+          *vv = nullptr, *attg = nullptr, *x1 = nullptr, *x3 = nullptr, *hg = nullptr, *logits = nullptr;
     int32_t *dtok = nullptr, *dpos = nullptr;
     unsigned long long *amax = nullptr;
     int32_t *dprompt = nullptr, *dout_ids = nullptr;
@@ -284,7 +287,33 @@ struct l2_model {
     // scratch for the operator-level entry points
     float *op_x = nullptr, *op_xg = nullptr, *op_y = nullptr;
     size_t op_cap = 0;
+    // per-launch event timing, on only inside l2_decode_profile
+    struct ProfRec { int cls; hipEvent_t e0, e1; };
+    bool prof_on = false;
+    std::vector<ProfRec> prof;
 };
+
+enum { K_EMBED = 0, K_Q4_QKV, K_ROPE_KV, K_ATTENTION, K_Q4_WO, K_Q4_W13, K_Q4_W2, K_CLASSIFIER, K_NEXT_TOKEN,
+       K_NCLASS };
+static const char *const kClassNames[K_NCLASS] = {"embed", "q4_qkv", "rope_kv", "attention", "q4_wo",
+                                                  "q4_w13", "q4_w2", "classifier", "next_token"};
+static constexpr int kMaxSplits = 64;
+
+// Time one launch with a pair of events on the launch stream (profiling runs only).
+#define LAUNCH(cls_, call)                                          \
+    do {                                                            \
+        if (m->prof_on) {                                           \
+            l2_model::ProfRec r_{cls_, nullptr, nullptr};           \
+            L2_HIP(hipEventCreate(&r_.e0));                         \
+            L2_HIP(hipEventCreate(&r_.e1));                         \
+            L2_HIP(hipEventRecord(r_.e0, m->stream));               \
+            L2_TRY(call);                                           \
+            L2_HIP(hipEventRecord(r_.e1, m->stream));               \
+            m->prof.push_back(r_);                                  \
+        } else {                                                    \
+            L2_TRY(call);                                           \
+        }                                                           \
+    } while (0)
 
 struct l2_state {
     l2_model *m = nullptr;
@@ -452,6 +481,26 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
         for (const Pending &p : pend) m->q[p.proj][p.layer].inv_index = m->dinv + p.inv_off;
     }
 
+    // Norm weights re-ordered for each consumer of a normalised vector, so that the
+    // matvec prologue reads them linearly: wn_c[j] = w[g_index_c[j]].
+    {
+        const size_t per_layer = (size_t)5 * dim;
+        std::vector<float> wn((size_t)L * per_layer);
+        const float *att_h = (const float *)(weights + ((const char *)m->rms_att - dbase));
+        const float *ffn_h = (const float *)(weights + ((const char *)m->rms_ffn - dbase));
+        const int projs[5] = {L2_WQ, L2_WK, L2_WV, L2_W1, L2_W3};
+        for (int l = 0; l < L; l++)
+            for (int c = 0; c < 5; c++) {
+                const float *src = (c < 3 ? att_h : ffn_h) + (size_t)l * dim;
+                const int32_t *g = (const int32_t *)(weights + ((const char *)m->q[projs[c]][l].g_index - dbase));
+                float *dst = wn.data() + l * per_layer + (size_t)c * dim;
+                for (int j = 0; j < dim; j++) dst[j] = src[g[j]];
+            }
+        M_TRY(dalloc(&m->dwn, wn.size()));
+        M_HIP(hipMemcpy(m->dwn, wn.data(), wn.size() * 4, hipMemcpyHostToDevice));
+        M_TRY(dalloc(&m->attn_part, (size_t)dims->n_heads * kMaxSplits * 130));
+    }
+
     // RoPE angles exactly as the reference evaluates them per element
     // (src/models.rs:107-110), computed once with the host's libm.
     {
@@ -530,9 +579,9 @@ extern "C" int l2_model_open(const char *path, const l2_dims *expect, int max_se
 extern "C" void l2_model_close(l2_model *m) {
     if (!m) return;
     if (m->stream) (void)hipStreamSynchronize(m->stream);
-    void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->x, m->xq, m->xk, m->xv, m->qv,
-                    m->kv, m->vv, m->attg, m->x1, m->x3, m->hb, m->hb2, m->hg, m->fin, m->logits,
-                    m->dtok, m->dpos, m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y};
+    void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->dwn, m->attn_part, m->x, m->xq, m->xk,
+                    m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->logits, m->dtok, m->dpos,
+                    m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y};
     for (void *p : ptrs) dfree(p);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
@@ -564,8 +613,7 @@ extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
 static int ensure_batch(l2_model *m, int B) {
     if (B <= m->cap_B) return L2_OK;
     L2_HIP(hipStreamSynchronize(m->stream));
-    float **bufs[] = {&m->x, &m->xq, &m->xk, &m->xv, &m->qv, &m->kv, &m->vv, &m->attg,
-                      &m->x1, &m->x3, &m->hb, &m->hb2, &m->hg, &m->fin};
+    float **bufs[] = {&m->x, &m->xq, &m->xk, &m->xv, &m->qv, &m->kv, &m->vv, &m->attg, &m->x1, &m->x3, &m->hg};
     for (float **b : bufs) {
         dfree(*b);
         *b = nullptr;
@@ -585,10 +633,7 @@ static int ensure_batch(l2_model *m, int B) {
     L2_TRY(dalloc(&m->attg, B * dim));
     L2_TRY(dalloc(&m->x1, B * dim));
     L2_TRY(dalloc(&m->x3, B * dim));
-    L2_TRY(dalloc(&m->hb, B * hid));
-    L2_TRY(dalloc(&m->hb2, B * hid));
     L2_TRY(dalloc(&m->hg, B * hid));
-    L2_TRY(dalloc(&m->fin, B * dim));
     L2_TRY(dalloc(&m->dtok, (size_t)B));
     L2_TRY(dalloc(&m->dpos, (size_t)B));
     if (!m->logits) L2_TRY(dalloc(&m->logits, (size_t)m->d.vocab_size));
@@ -665,31 +710,34 @@ extern "C" int l2_state_fill_synthetic(l2_state *s, int pos0, int npos, uint64_t
 // ---------------------------------------------------------------------------
 // operators
 
-static Q4Mat mat_of(const DevQLinear &q, const float *x, float *y, int y_stride, const float *res,
-                    const int32_t *scatter) {
+static Q4Mat mat_of(const DevQLinear &q, const float *x, const float *wn, float *y) {
     Q4Mat M{};
     M.qweight = q.qweight;
     M.qzeros = q.qzeros;
     M.scales = q.scales;
     M.x = x;
+    M.wn = wn;
     M.y = y;
-    M.res = res;
-    M.scatter = scatter;
     M.out = q.out;
-    M.y_stride = y_stride;
     return M;
 }
 
-static int q4_one(const DevQLinear &q, const float *xg, float *y, const float *res, const int32_t *scatter,
-                  int B, hipStream_t st) {
+static Q4Launch launch_of(const DevQLinear &q, int B, float eps) {
     Q4Launch L{};
-    L.m[0] = mat_of(q, xg, y, q.out, res, scatter);
     L.n_mats = 1;
     L.in = q.in;
     L.groups = q.groups;
     L.group_size = q.group_size;
-    L.epi = res ? Q4_EPI_RESIDUAL : Q4_EPI_STORE;
     L.batch = B;
+    L.eps = eps;
+    L.e.kind = Q4_EPI_STORE;
+    return L;
+}
+
+// y = W xg for one matrix, plain store.
+static int q4_one(const DevQLinear &q, const float *xg, float *y, int B, hipStream_t st) {
+    Q4Launch L = launch_of(q, B, 0.f);
+    L.m[0] = mat_of(q, xg, nullptr, y);
     return q4_matvec_launch(L, st);
 }
 
@@ -769,7 +817,7 @@ static int matvec_host(const DevQLinear &q, float *dx, float *dxg, float *dy, co
                        float *y_host, hipStream_t st) {
     L2_HIP(hipMemcpyAsync(dx, x_host, (size_t)B * q.in * 4, hipMemcpyHostToDevice, st));
     L2_TRY(gather_launch(dxg, dx, q.g_index, q.in, B, st));
-    L2_TRY(q4_one(q, dxg, dy, nullptr, nullptr, B, st));
+    L2_TRY(q4_one(q, dxg, dy, B, st));
     L2_HIP(hipMemcpyAsync(y_host, dy, (size_t)B * q.out * 4, hipMemcpyDeviceToHost, st));
     L2_HIP(hipStreamSynchronize(st));
     return L2_OK;
@@ -811,7 +859,7 @@ extern "C" int l2_model_classifier(l2_model *m, const float *x_host, float *y_ho
     if (!m || !x_host || !y_host) return l2_fail(L2_ERR_ARG, "null argument");
     L2_TRY(op_scratch(m, (size_t)std::max(m->d.dim, m->d.vocab_size)));
     L2_HIP(hipMemcpyAsync(m->op_x, x_host, (size_t)m->d.dim * 4, hipMemcpyHostToDevice, m->stream));
-    L2_TRY(dense_matvec_launch(m->op_y, m->wcls, m->op_x, m->d.dim, m->d.vocab_size, nullptr, m->stream));
+    L2_TRY(dense_matvec_launch(m->op_y, m->wcls, m->op_x, nullptr, 0.f, m->d.dim, m->d.vocab_size, nullptr, m->stream));
     L2_HIP(hipMemcpyAsync(y_host, m->op_y, (size_t)m->d.vocab_size * 4, hipMemcpyDeviceToHost, m->stream));
     L2_HIP(hipStreamSynchronize(m->stream));
     return L2_OK;
@@ -823,73 +871,111 @@ extern "C" int l2_model_classifier(l2_model *m, const float *x_host, float *y_ho
 // Enqueue one forward pass for the B tokens / positions already in m->dtok /
 // m->dpos.  max_pos is the largest position among them (sizes the attention
 // scratch).  With want_logits the classifier and the running argmax follow.
+//
+// Five launches per layer when B == 1: q|k|v with the attention rmsnorm in
+// front; attention with RoPE and the cache write folded in; wo with the
+// residual add behind; w1|w3 with the ffn rmsnorm in front and the SiLU gate
+// behind; w2 with the residual add behind.  Every producer writes its result
+// in the input order (g_index) of whoever reads it next.
 static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits) {
     const l2_dims &d = m->d;
     const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
     hipStream_t st = m->stream;
-    L2_TRY(embed_launch(m->x, m->tok_emb, m->dtok, dim, d.vocab_size, B, st)); // :189-191
+    {   // :189-191
+        ScatterTargets t{};
+        t.n = 3;
+        t.inv[0] = m->q[L2_WQ][0].inv_index, t.inv[1] = m->q[L2_WK][0].inv_index, t.inv[2] = m->q[L2_WV][0].inv_index;
+        t.out[0] = m->xq, t.out[1] = m->xk, t.out[2] = m->xv;
+        LAUNCH(K_EMBED, embed_launch(m->x, m->tok_emb, m->dtok, dim, B, t, m->amax, st));
+    }
     for (int l = 0; l < L; l++) {
         const DevQLinear &wq = m->q[L2_WQ][l], &wk = m->q[L2_WK][l], &wv = m->q[L2_WV][l],
                          &wo = m->q[L2_WO][l], &w1 = m->q[L2_W1][l], &w2 = m->q[L2_W2][l],
                          &w3 = m->q[L2_W3][l];
-        // attention rmsnorm (:217-219), delivered in the three input orders
-        ScatterTargets t{};
-        t.n = 3;
-        t.inv[0] = wq.inv_index, t.inv[1] = wk.inv_index, t.inv[2] = wv.inv_index;
-        t.out[0] = m->xq, t.out[1] = m->xk, t.out[2] = m->xv;
-        L2_TRY(rmsnorm_scatter_launch(m->x, m->rms_att + (size_t)l * dim, m->rms_eps, dim, B, t, st));
-        {   // q, k, v (:224-226) in one launch
-            Q4Launch Q{};
-            Q.m[0] = mat_of(wq, m->xq, m->qv, dim, nullptr, nullptr);
-            Q.m[1] = mat_of(wk, m->xk, m->kv, kvd, nullptr, nullptr);
-            Q.m[2] = mat_of(wv, m->xv, m->vv, kvd, nullptr, nullptr);
+        const float *wn = m->dwn + (size_t)l * 5 * dim;
+        {   // attention rmsnorm (:217-219) + q, k, v (:224-226)
+            Q4Launch Q = launch_of(wq, B, m->rms_eps);
+            Q.m[0] = mat_of(wq, m->xq, wn + 0 * (size_t)dim, m->qv);
+            Q.m[1] = mat_of(wk, m->xk, wn + 1 * (size_t)dim, m->kv);
+            Q.m[2] = mat_of(wv, m->xv, wn + 2 * (size_t)dim, m->vv);
             Q.n_mats = 3;
-            Q.in = dim;
-            Q.groups = wq.groups;
-            Q.group_size = d.group_size;
-            Q.epi = Q4_EPI_STORE;
-            Q.batch = B;
-            L2_TRY(q4_matvec_launch(Q, st));
+            LAUNCH(K_Q4_QKV, q4_matvec_launch(Q, st));
         }
         float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
         float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
-        // rope + cache write for all B columns (:228-249), then attention (:250-256)
-        L2_TRY(rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
-                              d.n_kv_heads, m->head_size, B, st));
-        L2_TRY(attention_launch(m->attg, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
-                                m->head_size, max_pos, B, st));
-        // wo and the residual (:260-264)
-        L2_TRY(q4_one(wo, m->attg, m->x, m->x, nullptr, B, st));
-        // ffn rmsnorm (:266), w1 | w3 (:271-272), silu gate (:274-276), w2 + residual (:279-285)
-        ScatterTargets t2{};
-        t2.n = 2;
-        t2.inv[0] = w1.inv_index, t2.inv[1] = w3.inv_index;
-        t2.out[0] = m->x1, t2.out[1] = m->x3;
-        L2_TRY(rmsnorm_scatter_launch(m->x, m->rms_ffn + (size_t)l * dim, m->rms_eps, dim, B, t2, st));
-        {
-            Q4Launch Q{};
-            Q.m[0] = mat_of(w1, m->x1, m->hb, hid, nullptr, nullptr);
-            Q.m[1] = mat_of(w3, m->x3, m->hb2, hid, nullptr, nullptr);
-            Q.n_mats = 2;
-            Q.in = dim;
-            Q.groups = w1.groups;
-            Q.group_size = d.group_size;
-            Q.epi = Q4_EPI_STORE;
-            Q.batch = B;
-            L2_TRY(q4_matvec_launch(Q, st));
+        if (B == 1) { // rope (:228-230), cache write (:236-249), attention (:250-256)
+            AttnDecode a{};
+            a.q = m->qv, a.k_new = m->kv, a.v_new = m->vv;
+            a.kcache = kc, a.vcache = vc;
+            a.cos_t = m->rope_cos, a.sin_t = m->rope_sin;
+            a.dpos = m->dpos;
+            a.out = m->attg, a.scatter = wo.inv_index;
+            a.part = m->attn_part;
+            a.n_heads = d.n_heads, a.n_kv_heads = d.n_kv_heads;
+            a.max_splits = kMaxSplits;
+            const int n_t = max_pos + 1;
+            if (n_t <= 256) {
+                a.ts = 256;
+                a.n_splits = 1;
+            } else {
+                // enough blocks to cover the CUs, at least 64 timesteps each
+                int want = (256 + d.n_kv_heads - 1) / d.n_kv_heads;
+                if (want > kMaxSplits) want = kMaxSplits;
+                int ts = ((n_t + want - 1) / want + 63) / 64 * 64;
+                const int qg = d.n_heads / d.n_kv_heads;
+                while ((size_t)ts * qg * 4 > 32 * 1024) ts -= 64;
+                if (ts < 64) ts = 64;
+                a.ts = ts;
+                a.n_splits = (n_t + ts - 1) / ts;
+                if (a.n_splits > kMaxSplits)
+                    return l2_fail(L2_ERR_RANGE, "attention: position %d needs %d splits", max_pos, a.n_splits);
+            }
+            LAUNCH(K_ATTENTION, attention_decode_launch(a, st));
+        } else {
+            LAUNCH(K_ROPE_KV, rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
+                                             d.n_kv_heads, m->head_size, B, st));
+            LAUNCH(K_ATTENTION, attention_launch(m->attg, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads,
+                                                 d.n_kv_heads, m->head_size, max_pos, B, st));
         }
-        L2_TRY(silu_scatter_launch(m->hg, m->hb, m->hb2, w2.inv_index, hid, B, st));
-        L2_TRY(q4_one(w2, m->hg, m->x, m->x, nullptr, B, st));
+        {   // wo (:260) + residual (:263-264); the new x also goes out in w1's and w3's order
+            Q4Launch Q = launch_of(wo, B, 0.f);
+            Q.m[0] = mat_of(wo, m->attg, nullptr, m->x);
+            Q.e.kind = Q4_EPI_RESIDUAL;
+            Q.e.res = m->x;
+            Q.e.n_scatter = 2;
+            Q.e.sc_idx[0] = w1.inv_index, Q.e.sc_out[0] = m->x1;
+            Q.e.sc_idx[1] = w3.inv_index, Q.e.sc_out[1] = m->x3;
+            LAUNCH(K_Q4_WO, q4_matvec_launch(Q, st));
+        }
+        {   // ffn rmsnorm (:266) + w1 | w3 (:271-272) + silu gate (:274-276), in w2's order
+            Q4Launch Q = launch_of(w1, B, m->rms_eps);
+            Q.m[0] = mat_of(w1, m->x1, wn + 3 * (size_t)dim, nullptr);
+            Q.m[1] = mat_of(w3, m->x3, wn + 4 * (size_t)dim, nullptr);
+            Q.n_mats = 2;
+            Q.pair = 1;
+            Q.e.kind = Q4_EPI_SCATTER_ONLY;
+            Q.e.n_scatter = 1;
+            Q.e.sc_idx[0] = w2.inv_index, Q.e.sc_out[0] = m->hg;
+            LAUNCH(K_Q4_W13, q4_matvec_launch(Q, st));
+        }
+        {   // w2 (:279) + residual (:283-285); the new x goes out in the next layer's q, k, v order
+            Q4Launch Q = launch_of(w2, B, 0.f);
+            Q.m[0] = mat_of(w2, m->hg, nullptr, m->x);
+            Q.e.kind = Q4_EPI_RESIDUAL;
+            Q.e.res = m->x;
+            if (l + 1 < L) {
+                Q.e.n_scatter = 3;
+                Q.e.sc_idx[0] = m->q[L2_WQ][l + 1].inv_index, Q.e.sc_out[0] = m->xq;
+                Q.e.sc_idx[1] = m->q[L2_WK][l + 1].inv_index, Q.e.sc_out[1] = m->xk;
+                Q.e.sc_idx[2] = m->q[L2_WV][l + 1].inv_index, Q.e.sc_out[2] = m->xv;
+            }
+            LAUNCH(K_Q4_W2, q4_matvec_launch(Q, st));
+        }
+        (void)hid;
     }
-    if (want_logits) { // :288-297, B == 1 only
-        ScatterTargets t{};
-        t.n = 1;
-        t.inv[0] = nullptr;
-        t.out[0] = m->fin;
-        L2_TRY(rmsnorm_scatter_launch(m->x, m->rms_final, m->rms_eps, dim, 1, t, st));
-        L2_TRY(fill_u64_launch(m->amax, 0ull, 1, st));
-        L2_TRY(dense_matvec_launch(m->logits, m->wcls, m->fin, dim, d.vocab_size, m->amax, st));
-    }
+    if (want_logits) // final rmsnorm + classifier (:288-297, B == 1 only) + running argmax
+        LAUNCH(K_CLASSIFIER, dense_matvec_launch(m->logits, m->wcls, m->x, m->rms_final, m->rms_eps, dim,
+                                                 d.vocab_size, m->amax, st));
     return L2_OK;
 }
 
@@ -966,7 +1052,7 @@ static int ensure_loop_buffers(l2_model *m, int n_prompt, int n_out) {
 // token, and the device position advanced.
 static int loop_step(l2_model *m, l2_state *s, int pos, int n_prompt, int pos0) {
     L2_TRY(forward_enqueue(m, s, 1, pos, true));
-    L2_TRY(next_token_launch(m->amax, m->dprompt, n_prompt, m->dpos, m->dout_ids, pos0, m->dtok, m->stream));
+    LAUNCH(K_NEXT_TOKEN, next_token_launch(m->amax, m->dprompt, n_prompt, m->dpos, m->dout_ids, pos0, m->dtok, m->stream));
     return L2_OK;
 }
 
@@ -1035,12 +1121,12 @@ extern "C" int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_tot
     hipEvent_t e0, e1;
     L2_HIP(hipEventCreate(&e0));
     L2_HIP(hipEventCreate(&e1));
-    for (int i = 0; i < n; i++) L2_TRY(q4_one(qs[i]->q, qs[i]->xg, qs[i]->y, nullptr, nullptr, 1, st)); // warm-up
+    for (int i = 0; i < n; i++) L2_TRY(q4_one(qs[i]->q, qs[i]->xg, qs[i]->y, 1, st)); // warm-up
     L2_HIP(hipStreamSynchronize(st));
     L2_HIP(hipEventRecord(e0, st));
     for (int it = 0; it < iters; it++) {
         l2_qlinear *q = qs[it % n];
-        L2_TRY(q4_one(q->q, q->xg, q->y, nullptr, nullptr, 1, st));
+        L2_TRY(q4_one(q->q, q->xg, q->y, 1, st));
     }
     L2_HIP(hipEventRecord(e1, st));
     L2_HIP(hipEventSynchronize(e1));
@@ -1071,6 +1157,45 @@ extern "C" int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t 
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (out_ids) L2_HIP(hipMemcpy(out_ids, m->dout_ids, (size_t)n_tokens * 4, hipMemcpyDeviceToHost));
+    return L2_OK;
+}
+
+extern "C" int l2_kernel_class_count(void) { return K_NCLASS; }
+
+extern "C" const char *l2_kernel_class_name(int cls) { return cls >= 0 && cls < K_NCLASS ? kClassNames[cls] : ""; }
+
+extern "C" int l2_decode_profile(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
+                                 float *ms_by_class, int32_t *launches_by_class) {
+    if (!m || !s || !ms_by_class || !launches_by_class || n_tokens < 1) return l2_fail(L2_ERR_ARG, "bad argument");
+    if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
+    if (pos < 0 || pos + n_tokens > m->max_seq) return l2_fail(L2_ERR_RANGE, "positions [%d,%d) exceed the cache", pos, pos + n_tokens);
+    if (token < 0 || token >= m->d.vocab_size) return l2_fail(L2_ERR_RANGE, "token %d", token);
+    L2_TRY(ensure_batch(m, 1));
+    L2_TRY(ensure_loop_buffers(m, 1, n_tokens));
+    L2_TRY(set_i32_launch(m->dtok, token, m->dpos, pos, m->stream));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    m->prof.clear();
+    m->prof_on = true;
+    int rc = L2_OK;
+    for (int i = 0; i < n_tokens && rc == L2_OK; i++) rc = loop_step(m, s, pos + i, 0, pos);
+    m->prof_on = false;
+    hipError_t e = hipStreamSynchronize(m->stream);
+    for (int c = 0; c < K_NCLASS; c++) {
+        ms_by_class[c] = 0.f;
+        launches_by_class[c] = 0;
+    }
+    for (auto &r : m->prof) {
+        float ms = 0.f;
+        if (rc == L2_OK && e == hipSuccess && r.e0 && r.e1 && hipEventElapsedTime(&ms, r.e0, r.e1) == hipSuccess) {
+            ms_by_class[r.cls] += ms;
+            launches_by_class[r.cls] += 1;
+        }
+        if (r.e0) (void)hipEventDestroy(r.e0);
+        if (r.e1) (void)hipEventDestroy(r.e1);
+    }
+    m->prof.clear();
+    if (rc != L2_OK) return rc;
+    if (e != hipSuccess) return l2_fail(L2_ERR_HIP, "profile run: %s", hipGetErrorString(e));
     return L2_OK;
 }
 

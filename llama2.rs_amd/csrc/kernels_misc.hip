@@ -1,6 +1,7 @@
-// The per-token kernels around the q4 matvec: embedding gather, RMSNorm, RoPE +
-// KV-cache write, GQA attention, SiLU gate, the fp32 classifier with a fused
-// argmax, and the greedy loop's token hand-over.  gfx950, wave64.
+// The per-token kernels around the q4 matvec: embedding gather, RoPE + KV-cache
+// write, GQA attention (a split-KV decode kernel with RoPE folded in, and a
+// batched one for prefill chunks), the fp32 classifier with RMSNorm in front
+// and the argmax behind, and the greedy loop's token hand-over.  gfx950, wave64.
 //
 // This file is compiled with -ffp-contract=off: wherever the reference rounds
 // a product before adding (Rust never fuses), so does this code; FMAs appear
@@ -63,34 +64,19 @@ __device__ __forceinline__ float block_max(float v, float *red) {
     return s;
 }
 
-// x[b] = token_embedding_table[token[b]]  (src/models.rs:189-191)
-__global__ void embed_kernel(float *x, const float *emb, const int32_t *tokens, int dim) {
+// x[b] = token_embedding_table[token[b]]  (src/models.rs:189-191), also written
+// in the input order of the first layer's q, k and v projections.  Starts a
+// forward pass, so it also clears the running argmax.
+__global__ void embed_kernel(float *x, const float *emb, const int32_t *tokens, int dim, ScatterTargets t,
+                             unsigned long long *amax) {
     const int b = blockIdx.x;
-    const float4 *src = reinterpret_cast<const float4 *>(emb + (size_t)tokens[b] * dim);
-    float4 *dst = reinterpret_cast<float4 *>(x + (size_t)b * dim);
-    for (int i = threadIdx.x; i < dim / 4; i += blockDim.x) dst[i] = src[i];
-}
-
-// rmsnorm (src/models.rs:53-66): o[j] = (w[j] * ss) * x[j], ss = 1/sqrt(mean(x^2) + eps),
-// written through up to three inverse permutations.
-__global__ __launch_bounds__(1024) void rmsnorm_scatter_kernel(const float *x, const float *w, float eps,
-                                                                int dim, ScatterTargets t) {
-    __shared__ float red[16];
-    const int b = blockIdx.x;
-    const float *xb = x + (size_t)b * dim;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) ss = fmaf(xb[i], xb[i], ss);
-    ss = block_sum(ss, red);
-    ss /= (float)dim;
-    ss += eps;
-    ss = 1.0f / sqrtf(ss);
+    const float *src = emb + (size_t)tokens[b] * dim;
     for (int i = threadIdx.x; i < dim; i += blockDim.x) {
-        const float v = w[i] * ss * xb[i];
-        for (int c = 0; c < t.n; c++) {
-            const int dst = t.inv[c] ? t.inv[c][i] : i;
-            t.out[c][(size_t)b * dim + dst] = v;
-        }
+        const float v = src[i];
+        x[(size_t)b * dim + i] = v;
+        for (int c = 0; c < t.n; c++) t.out[c][(size_t)b * dim + t.inv[c][i]] = v;
     }
+    if (amax && b == 0 && threadIdx.x == 0) amax[0] = 0ull;
 }
 
 // out[b][j] = x[b][g_index[j]]  (src/gptq.rs:110-114), for callers that hand the
@@ -140,9 +126,10 @@ __global__ void rope_kv_kernel(float *q, const float *k, const float *v, const i
     for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) vc[i] = vb[i];
 }
 
-// multihead_attention (src/models.rs:131-176) for one (head, batch column):
-// scores over t = 0..=pos against the kv head h / attn_groups, softmax with
-// max subtraction and division by the sum (:68-81), then the weighted sum of V.
+// multihead_attention (src/models.rs:131-176) for one (head, batch column) of a
+// prefill chunk whose cache rows are already written: scores over t = 0..=pos
+// against the kv head h / attn_groups, softmax with max subtraction and
+// division by the sum (:68-81), then the weighted sum of V.
 // Dynamic LDS: att[pos+1].  head_size must be 128.
 __global__ __launch_bounds__(256) void attention_kernel(float *out, const float *q, const float *kcache,
                                                          const float *vcache, const int32_t *pos,
@@ -160,7 +147,7 @@ __global__ __launch_bounds__(256) void attention_kernel(float *out, const float 
     const int tid = threadIdx.x;
     if (tid < HS) qs[tid] = q[(size_t)b * dim + h * HS + tid];
     __syncthreads();
-    const float inv_div = sqrtf((float)HS);
+    const float root = sqrtf((float)HS);
     // scores: 4 lanes per timestep, 32 dims each
     const int sub = tid & 3;
     for (int t = tid >> 2; t <= p; t += 64) {
@@ -177,7 +164,7 @@ __global__ __launch_bounds__(256) void attention_kernel(float *out, const float 
         }
         s += dpp_xchg<0xB1>(s);
         s += dpp_xchg<0x4E>(s);
-        if (sub == 0) att[t] = s / inv_div;
+        if (sub == 0) att[t] = s / root;
     }
     __syncthreads();
     float m = -INFINITY;
@@ -195,6 +182,7 @@ __global__ __launch_bounds__(256) void attention_kernel(float *out, const float 
     // weighted values: thread -> (dim d, parity of t)
     const int d = tid & (HS - 1), par = tid >> 7;
     float acc = 0.f;
+#pragma unroll 4
     for (int t = par; t <= p; t += 2)
         acc = fmaf(att[t], vcache[(size_t)t * kv_dim + kvh * HS + d], acc);
     if (par == 1) part[d] = acc;
@@ -207,17 +195,171 @@ __global__ __launch_bounds__(256) void attention_kernel(float *out, const float 
     }
 }
 
-// silu gate (src/models.rs:92-98): s = s * (1 / (1 + exp(-s))), then s = s * s2.
-__global__ void silu_scatter_kernel(float *out, const float *a, const float *b2, const int32_t *scatter,
-                                    int n) {
-    const int b = blockIdx.y;
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    float s = a[(size_t)b * n + i];
-    s = s * (1.0f / (1.0f + expf(-s)));
-    s = s * b2[(size_t)b * n + i];
-    const int dst = scatter ? scatter[i] : i;
-    out[(size_t)b * n + dst] = s;
+// ---------------------------------------------------------------------------
+// Decode attention: one query position, all q heads of one kv head per block,
+// the timesteps cut into splits across grid.y (src/models.rs:131-176 computed
+// as softmax over partial maxima, which is the same function).
+//
+// RoPE (src/models.rs:100-129) is applied to q as it is staged, and to the new
+// key on its way into the cache (:236-249); the block that owns t == pos is the
+// only writer of that cache row and uses the fresh values directly.
+
+template <int QG>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
+    constexpr int HS = 128, HALF = 64;
+    extern __shared__ float sc[]; // [QG][ts] scores -> exp(score - max)
+    __shared__ float qs[QG * HS];
+    __shared__ float knew[HS];
+    __shared__ float ml[QG][2];
+    __shared__ float half2[QG][HS];
+    const int kvh = blockIdx.x, sp = blockIdx.y;
+    const int pos = A.dpos[0];
+    const int t0 = sp * A.ts;
+    if (t0 > pos) return;
+    const int t1 = min(t0 + A.ts, pos + 1);
+    const int n = t1 - t0;
+    const int kv_dim = A.n_kv_heads * HS;
+    const int tid = threadIdx.x;
+    const float *ct = A.cos_t + (size_t)pos * HALF;
+    const float *st = A.sin_t + (size_t)pos * HALF;
+    for (int idx = tid; idx < QG * HALF; idx += 256) {
+        const int j = idx >> 6, i = idx & 63;
+        const float *qh = A.q + (size_t)(kvh * QG + j) * HS;
+        const float c = ct[i], s = st[i];
+        const float a = qh[i], b = qh[i + HALF];
+        const float first = a * c - b * s;
+        qs[j * HS + i] = first;
+        qs[j * HS + HALF + i] = b * c + first * s; // the in-place quirk: rotated first half
+    }
+    const bool owns_new = (t1 == pos + 1);
+    if (owns_new) {
+        if (tid < HALF) {
+            const float *kh = A.k_new + (size_t)kvh * HS;
+            const float c = ct[tid], s = st[tid];
+            const float a = kh[tid], b = kh[tid + HALF];
+            const float first = a * c - b * s;
+            const float second = b * c + first * s;
+            knew[tid] = first;
+            knew[tid + HALF] = second;
+            float *kc = A.kcache + (size_t)pos * kv_dim + kvh * HS;
+            kc[tid] = first;
+            kc[tid + HALF] = second;
+        } else if (tid >= 128) {
+            const int d = tid - 128;
+            A.vcache[(size_t)pos * kv_dim + kvh * HS + d] = A.v_new[(size_t)kvh * HS + d];
+        }
+    }
+    __syncthreads();
+
+    // scores: 4 lanes per timestep, 32 dims each, all QG heads against one load of K
+    const int sub = tid & 3;
+    const float root = sqrtf((float)HS);
+    for (int tt = tid >> 2; tt < n; tt += 64) {
+        const int t = t0 + tt;
+        float4 kk[8];
+        if (t == pos) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) kk[i] = reinterpret_cast<const float4 *>(knew + sub * 32)[i];
+        } else {
+            const float4 *kr = reinterpret_cast<const float4 *>(A.kcache + (size_t)t * kv_dim + kvh * HS + sub * 32);
+#pragma unroll
+            for (int i = 0; i < 8; i++) kk[i] = kr[i];
+        }
+#pragma unroll
+        for (int j = 0; j < QG; j++) {
+            const float4 *qr = reinterpret_cast<const float4 *>(qs + j * HS + sub * 32);
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float4 qq = qr[i];
+                s = fmaf(qq.x, kk[i].x, s);
+                s = fmaf(qq.y, kk[i].y, s);
+                s = fmaf(qq.z, kk[i].z, s);
+                s = fmaf(qq.w, kk[i].w, s);
+            }
+            s += dpp_xchg<0xB1>(s);
+            s += dpp_xchg<0x4E>(s);
+            if (sub == 0) sc[j * A.ts + tt] = s / root;
+        }
+    }
+    __syncthreads();
+
+    // per head: max, exp, sum (wave w takes heads w, w+4)
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int j = wave; j < QG; j += 4) {
+        float *row = sc + j * A.ts;
+        float m = -INFINITY;
+        for (int tt = lane; tt < n; tt += 64) m = fmaxf(m, row[tt]);
+        m = wave_max(m);
+        float l = 0.f;
+        for (int tt = lane; tt < n; tt += 64) {
+            const float e = expf(row[tt] - m);
+            row[tt] = e;
+            l += e;
+        }
+        l = wave_sum(l);
+        if (lane == 0) {
+            ml[j][0] = m;
+            ml[j][1] = l;
+        }
+    }
+    __syncthreads();
+
+    // weighted values: thread -> (dim d, parity of t)
+    const int d = tid & (HS - 1), par = tid >> 7;
+    float acc[QG];
+#pragma unroll
+    for (int j = 0; j < QG; j++) acc[j] = 0.f;
+    const float *vbase = A.vcache + (size_t)kvh * HS + d;
+#pragma unroll 4
+    for (int tt = par; tt < n; tt += 2) {
+        const int t = t0 + tt;
+        const float v = (t == pos) ? A.v_new[(size_t)kvh * HS + d] : vbase[(size_t)t * kv_dim];
+#pragma unroll
+        for (int j = 0; j < QG; j++) acc[j] = fmaf(sc[j * A.ts + tt], v, acc[j]);
+    }
+    if (par == 1) {
+#pragma unroll
+        for (int j = 0; j < QG; j++) half2[j][d] = acc[j];
+    }
+    __syncthreads();
+    if (par == 0) {
+#pragma unroll
+        for (int j = 0; j < QG; j++) {
+            const float o = acc[j] + half2[j][d];
+            const int h = kvh * QG + j;
+            if (A.n_splits == 1) {
+                const int i = h * HS + d;
+                A.out[A.scatter ? A.scatter[i] : i] = o / ml[j][1];
+            } else {
+                float *p = A.part + ((size_t)h * A.max_splits + sp) * (HS + 2);
+                p[d] = o;
+                if (d == 0) {
+                    p[HS] = ml[j][0];
+                    p[HS + 1] = ml[j][1];
+                }
+            }
+        }
+    }
+}
+
+// Merge the splits of one q head: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s.
+__global__ __launch_bounds__(128) void attn_combine_kernel(const AttnDecode A) {
+    constexpr int HS = 128;
+    const int h = blockIdx.x, d = threadIdx.x;
+    const int pos = A.dpos[0];
+    const int ns = min(A.n_splits, pos / A.ts + 1);
+    const float *p = A.part + (size_t)h * A.max_splits * (HS + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < ns; s++) M = fmaxf(M, p[s * (HS + 2) + HS]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < ns; s++) {
+        const float w = expf(p[s * (HS + 2) + HS] - M);
+        num = fmaf(w, p[s * (HS + 2) + d], num);
+        den = fmaf(w, p[s * (HS + 2) + HS + 1], den);
+    }
+    const int i = h * HS + d;
+    A.out[A.scatter ? A.scatter[i] : i] = num / den;
 }
 
 // Order-preserving key for (value, index): larger value wins, equal values ->
@@ -230,14 +372,39 @@ __device__ __forceinline__ unsigned long long amax_key(float v, int idx) {
 }
 
 // Linear::matvec (src/model.rs:22-31) for the classifier: one wave per row,
-// two rows in flight, x staged in LDS.  Optionally folds each logit into a
-// 64-bit (value,index) maximum.
-__global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float *w, const float *x, int in,
-                                                            int out, unsigned long long *amax) {
+// two rows in flight, x staged in LDS.  With wn set, x is first normalised as
+// rmsnorm does (src/models.rs:53-66, :288-295): the block stages wn[i]*x[i] and
+// scales each logit by ss = 1/sqrt(mean(x^2) + eps).  Optionally folds each
+// logit into a 64-bit (value,index) maximum.
+__global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float *w, const float *x,
+                                                            const float *wn, float eps, int in, int out,
+                                                            unsigned long long *amax) {
     extern __shared__ float xs[];
+    __shared__ float red[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < in / 4; i += 256)
-        reinterpret_cast<float4 *>(xs)[i] = reinterpret_cast<const float4 *>(x)[i];
+    float ssq = 0.f;
+    for (int i = tid; i < in / 4; i += 256) {
+        float4 v = reinterpret_cast<const float4 *>(x)[i];
+        if (wn) {
+            const float4 g = reinterpret_cast<const float4 *>(wn)[i];
+            ssq = fmaf(v.x, v.x, ssq);
+            ssq = fmaf(v.y, v.y, ssq);
+            ssq = fmaf(v.z, v.z, ssq);
+            ssq = fmaf(v.w, v.w, ssq);
+            v.x *= g.x;
+            v.y *= g.y;
+            v.z *= g.z;
+            v.w *= g.w;
+        }
+        reinterpret_cast<float4 *>(xs)[i] = v;
+    }
+    float ss = 1.0f;
+    if (wn) {
+        ssq = block_sum(ssq, red);
+        ssq /= (float)in;
+        ssq += eps;
+        ss = 1.0f / sqrtf(ssq);
+    }
     __syncthreads();
     const int n4 = in / 4;
     const int waves_total = gridDim.x * 4;
@@ -246,6 +413,7 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float
         const float4 *r0 = reinterpret_cast<const float4 *>(w + (size_t)o * in);
         const float4 *r1 = reinterpret_cast<const float4 *>(w + (size_t)o1 * in);
         float a0 = 0.f, a1 = 0.f;
+#pragma unroll 4
         for (int j = lane; j < n4; j += 64) {
             const float4 xv = reinterpret_cast<const float4 *>(xs)[j];
             const float4 w0 = r0[j], w1 = r1[j];
@@ -258,8 +426,8 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float
             a1 = fmaf(w1.z, xv.z, a1);
             a1 = fmaf(w1.w, xv.w, a1);
         }
-        a0 = wave_sum(a0);
-        a1 = wave_sum(a1);
+        a0 = wave_sum(a0) * ss;
+        a1 = wave_sum(a1) * ss;
         if (lane == 0) {
             y[o] = a0;
             unsigned long long key = amax_key(a0, o);
@@ -271,11 +439,6 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float
             if (amax) atomicMax(amax, key);
         }
     }
-}
-
-__global__ void fill_u64_kernel(unsigned long long *p, unsigned long long v, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = v;
 }
 
 // Greedy hand-over (src/inference.rs:154-162, 185-189): next is the forced
@@ -311,19 +474,10 @@ __global__ void fill_pattern_kernel(float *p, size_t n, uint64_t seed) {
 
 } // namespace
 
-int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int vocab, int B,
-                 hipStream_t st) {
-    (void)vocab;
-    if (dim % 4) return l2_fail(L2_ERR_ARG, "embed: dim=%d not a multiple of 4", dim);
-    hipLaunchKernelGGL(embed_kernel, dim3(B), dim3(256), 0, st, x, emb, tokens, dim);
-    L2_HIP(hipGetLastError());
-    return L2_OK;
-}
-
-int rmsnorm_scatter_launch(const float *x, const float *w, float eps, int dim, int B,
-                           const ScatterTargets &t, hipStream_t st) {
-    if (t.n < 1 || t.n > 3) return l2_fail(L2_ERR_ARG, "rmsnorm: %d targets", t.n);
-    hipLaunchKernelGGL(rmsnorm_scatter_kernel, dim3(B), dim3(1024), 0, st, x, w, eps, dim, t);
+int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int B, const ScatterTargets &t,
+                 unsigned long long *amax_key, hipStream_t st) {
+    if (t.n < 0 || t.n > 3) return l2_fail(L2_ERR_ARG, "embed: %d targets", t.n);
+    hipLaunchKernelGGL(embed_kernel, dim3(B), dim3(1024), 0, st, x, emb, tokens, dim, t, amax_key);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }
@@ -355,26 +509,35 @@ int attention_launch(float *out, const float *q, const float *kcache_l, const fl
     return L2_OK;
 }
 
-int silu_scatter_launch(float *out, const float *a, const float *b, const int32_t *scatter, int n,
-                        int B, hipStream_t st) {
-    hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, a, b, scatter, n);
+int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
+    const int qg = a.n_heads / a.n_kv_heads;
+    if (a.ts < 64 || a.ts % 64 || a.n_splits < 1 || a.n_splits > a.max_splits)
+        return l2_fail(L2_ERR_ARG, "attention: ts=%d splits=%d/%d", a.ts, a.n_splits, a.max_splits);
+    const size_t lds = (size_t)qg * a.ts * sizeof(float);
+    if (lds > 40 * 1024) return l2_fail(L2_ERR_ARG, "attention: %d heads x %d timesteps per block", qg, a.ts);
+    dim3 grid(a.n_kv_heads, a.n_splits), block(256);
+    switch (qg) {
+        case 1: hipLaunchKernelGGL(attn_decode_kernel<1>, grid, block, lds, st, a); break;
+        case 2: hipLaunchKernelGGL(attn_decode_kernel<2>, grid, block, lds, st, a); break;
+        case 4: hipLaunchKernelGGL(attn_decode_kernel<4>, grid, block, lds, st, a); break;
+        case 8: hipLaunchKernelGGL(attn_decode_kernel<8>, grid, block, lds, st, a); break;
+        default: return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
+    }
     L2_HIP(hipGetLastError());
+    if (a.n_splits > 1) {
+        hipLaunchKernelGGL(attn_combine_kernel, dim3(a.n_heads), dim3(128), 0, st, a);
+        L2_HIP(hipGetLastError());
+    }
     return L2_OK;
 }
 
-int dense_matvec_launch(float *y, const float *w, const float *x, int in, int out,
+int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
                         unsigned long long *amax_key, hipStream_t st) {
     if (in % 4 || in * 4 > 64 * 1024) return l2_fail(L2_ERR_ARG, "dense matvec: in=%d", in);
     int blocks = (out + 7) / 8;
     if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(dense_matvec_kernel, dim3(blocks), dim3(256), (size_t)in * 4, st, y, w, x, in, out,
-                       amax_key);
-    L2_HIP(hipGetLastError());
-    return L2_OK;
-}
-
-int fill_u64_launch(unsigned long long *p, unsigned long long v, int n, hipStream_t st) {
-    hipLaunchKernelGGL(fill_u64_kernel, dim3((n + 255) / 256), dim3(256), 0, st, p, v, n);
+    hipLaunchKernelGGL(dense_matvec_kernel, dim3(blocks), dim3(256), (size_t)in * 4, st, y, w, x, wn, eps, in,
+                       out, amax_key);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }

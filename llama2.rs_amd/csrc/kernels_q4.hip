@@ -1,4 +1,5 @@
-// GPTQ 4-bit dequant matvec for gfx950 (wave64).
+// GPTQ 4-bit dequant matvec for gfx950 (wave64), with the neighbouring
+// element-wise steps of the decode schedule folded into its two ends.
 //
 // Computes, per output row o and batch column b (QLinear::matvec,
 // src/gptq.rs:94-176, in exact arithmetic):
@@ -16,11 +17,20 @@
 //
 // Arithmetic.  The zero point is factored out of the inner loop:
 //   sum_{j in chunk} s (n_j - z) x_j = s * (sum n_j x_j - z * sum x_j)
-// Nibbles are turned into floats by v_cvt_f32_ubyteN on words masked with
-// 0x0F0F0F0F (even nibbles) and 0xF0F0F0F0 (odd nibbles, scaled by 16, undone
-// exactly afterwards), so one nibble costs one convert and one FMA.  All
-// accumulation is fp32; the reduction order is fixed (no atomics), so results
-// are bit-stable from run to run.
+// Nibbles are turned into floats two at a time by v_cvt_pk_f32_fp8 (see
+// chunk_dot), so one nibble costs half a convert, one FMA and 3/8 of a mask
+// operation.  All accumulation is fp32; the reduction order is fixed (no
+// atomics), so results are bit-stable from run to run.
+//
+// Prologue (optional): rmsnorm (src/models.rs:53-66).  The input buffer then
+// holds the raw residual stream in this layer's g_index order and `wn` the norm
+// weights in the same order; the block stages wn[j]*x[j], sums x^2 on the way,
+// and applies ss = 1/sqrt(mean + eps) once per output row (W(ss v) = ss W v).
+//
+// Epilogues: plain store; residual add (src/models.rs:263-264, 283-285) that
+// also delivers the new residual stream in the input order of up to three
+// following layers; SiLU gate over a (w1, w3) pair of rows
+// (src/models.rs:271-276) delivered in w2's input order.
 #include "l2_internal.h"
 
 namespace {
@@ -44,175 +54,275 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// 32 nibbles of one row against 32 inputs.  lo collects even nibbles, hi the
-// odd ones times 16.
-__device__ __forceinline__ void chunk_dot(const uint4 w, const float (&x)[32], float &lo, float &hi) {
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+// 32 nibbles of one row against 32 inputs: returns 2^-9 * sum_k n_k x_k.
+//
+// A nibble n parked in the low half of a byte, 0000nnnn, read as an OCP FP8
+// E4M3 number is exactly n * 2^-9 (subnormal for n < 8, exponent 1 above, the
+// same step on both sides), so v_cvt_pk_f32_fp8 turns two nibbles into two
+// floats in one instruction.  Even nibbles come from w & 0x0F0F0F0F, odd ones
+// from (w >> 4) & 0x0F0F0F0F.  The power of two is undone exactly by the
+// caller.
+__device__ __forceinline__ float chunk_dot(const uint4 w, const float (&x)[32]) {
     const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+    float a0 = 0.f, a1 = 0.f;
 #pragma unroll
     for (int d = 0; d < 4; d++) {
         const uint32_t l = words[d] & 0x0F0F0F0Fu;
-        const uint32_t h = words[d] & 0xF0F0F0F0u;
-        lo = fmaf((float)(l & 0xFFu), x[8 * d + 0], lo);
-        hi = fmaf((float)(h & 0xFFu), x[8 * d + 1], hi);
-        lo = fmaf((float)((l >> 8) & 0xFFu), x[8 * d + 2], lo);
-        hi = fmaf((float)((h >> 8) & 0xFFu), x[8 * d + 3], hi);
-        lo = fmaf((float)((l >> 16) & 0xFFu), x[8 * d + 4], lo);
-        hi = fmaf((float)((h >> 16) & 0xFFu), x[8 * d + 5], hi);
-        lo = fmaf((float)(l >> 24), x[8 * d + 6], lo);
-        hi = fmaf((float)(h >> 24), x[8 * d + 7], hi);
+        const uint32_t h = (words[d] >> 4) & 0x0F0F0F0Fu;
+        const v2f l01 = __builtin_amdgcn_cvt_pk_f32_fp8(l, false); // nibbles 0, 2
+        const v2f l23 = __builtin_amdgcn_cvt_pk_f32_fp8(l, true);  // nibbles 4, 6
+        const v2f h01 = __builtin_amdgcn_cvt_pk_f32_fp8(h, false); // nibbles 1, 3
+        const v2f h23 = __builtin_amdgcn_cvt_pk_f32_fp8(h, true);  // nibbles 5, 7
+        a0 = fmaf(l01.x, x[8 * d + 0], a0);
+        a1 = fmaf(h01.x, x[8 * d + 1], a1);
+        a0 = fmaf(l01.y, x[8 * d + 2], a0);
+        a1 = fmaf(h01.y, x[8 * d + 3], a1);
+        a0 = fmaf(l23.x, x[8 * d + 4], a0);
+        a1 = fmaf(h23.x, x[8 * d + 5], a1);
+        a0 = fmaf(l23.y, x[8 * d + 6], a0);
+        a1 = fmaf(h23.y, x[8 * d + 7], a1);
     }
+    return a0 + a1;
 }
 
-// G: group size, R: rows per wave, NW: waves per block.
-template <int G, int R, int NW>
+// Stage one input vector into padded chunks + chunk sums; returns this
+// thread's share of sum(x^2) (of the raw input, before the norm weight).
+template <int NW>
+__device__ __forceinline__ float stage_input(const float *__restrict__ xin_f, const float *__restrict__ wn_f,
+                                             int in, float *xs, float *xsum, int tid) {
+    const float4 *xin = reinterpret_cast<const float4 *>(xin_f);
+    const float4 *wn = reinterpret_cast<const float4 *>(wn_f);
+    const int n4 = in >> 2;
+    constexpr int T = NW * 64, U = 4;
+    float ssq = 0.f;
+    for (int base = 0; base < n4; base += T * U) {
+        float4 v[U], g[U];
+        // all loads of a batch are issued before the first one is consumed
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int j4 = base + u * T + tid;
+            v[u] = j4 < n4 ? xin[j4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            g[u] = (wn_f && j4 < n4) ? wn[j4] : make_float4(1.f, 1.f, 1.f, 1.f);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int j4 = base + u * T + tid;
+            if (wn_f) {
+                ssq = fmaf(v[u].x, v[u].x, ssq);
+                ssq = fmaf(v[u].y, v[u].y, ssq);
+                ssq = fmaf(v[u].z, v[u].z, ssq);
+                ssq = fmaf(v[u].w, v[u].w, ssq);
+                v[u].x *= g[u].x;
+                v[u].y *= g[u].y;
+                v[u].z *= g[u].z;
+                v[u].w *= g[u].w;
+            }
+            // the 8 consecutive lanes that hold one chunk add up its sum
+            float s = (v[u].x + v[u].y) + (v[u].z + v[u].w);
+            s += dpp_xchg<0xB1>(s);  // lanes ^1
+            s += dpp_xchg<0x4E>(s);  // lanes ^2
+            s += dpp_xchg<0x141>(s); // 7 - lane within each 8: the other quad
+            if (j4 < n4) {
+                const int j = j4 << 2;
+                *reinterpret_cast<float4 *>(&xs[(j >> 5) * kChunkPad + (j & 31)]) = v[u];
+                if ((tid & 7) == 0) xsum[j >> 5] = s;
+            }
+        }
+    }
+    return ssq;
+}
+
+struct RowLoad {
+    uint4 w;
+    float s;
+};
+
+// G: group size, R: rows per wave (per matrix), NW: waves per block,
+// PAIR: the block walks rows of m[0] and m[1] together (SiLU gate).
+template <int G, int R, int NW, bool PAIR>
 __global__ __launch_bounds__(NW * 64) void q4_matvec_kernel(const Q4Launch L) {
     extern __shared__ float lds[];
+    constexpr int NM = PAIR ? 2 : 1;
     const int in = L.in;
-    const int C = in >> 5;             // chunks per row
-    float *xs = lds;                   // [C][36]
-    float *xsum = lds + C * kChunkPad; // [C]
+    const int C = in >> 5;                 // chunks per row
+    const int xstride = C * kChunkPad + C; // floats per staged vector: [C][36] then [C] sums
+    __shared__ float red[NW];
 
     // which matrix, which rows
     int rb = blockIdx.x;
     int mi = 0;
-    while (mi + 1 < L.n_mats && rb >= L.m[mi].row_blocks) {
-        rb -= L.m[mi].row_blocks;
-        mi++;
+    if (!PAIR) {
+        while (mi + 1 < L.n_mats && rb >= L.m[mi].row_blocks) {
+            rb -= L.m[mi].row_blocks;
+            mi++;
+        }
     }
-    const Q4Mat &M = L.m[mi];
     const int b = blockIdx.y;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int n_out = L.m[mi].out;
     const int o0 = (rb * NW + wave) * R; // first row of this wave; multiple of R
-    const bool active = o0 < M.out;
+    const bool active = o0 < n_out;
     const int groups = L.groups;
+    constexpr int CPG = G / 32; // chunks per group
 
     // First chunk's weights are requested before anything else so that the HBM
     // latency overlaps with staging x.
-    uint4 wcur[R];
-    float scur[R];
-    int32_t zcur = 0;
+    RowLoad cur[NM][R];
+    int32_t zcur[NM];
     int c = lane;
-    constexpr int CPG = G / 32; // chunks per group
     if (active && c < C) {
         const int g = c / CPG;
-        zcur = M.qzeros[(size_t)(o0 >> 3) * groups + g];
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int o = min(o0 + r, M.out - 1);
-            wcur[r] = M.qweight[(size_t)o * C + c];
-            scur[r] = M.scales[(size_t)o * groups + g];
+        for (int q = 0; q < NM; q++) {
+            const Q4Mat &M = L.m[mi + q];
+            zcur[q] = M.qzeros[(size_t)(o0 >> 3) * groups + g];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int o = min(o0 + r, n_out - 1);
+                cur[q][r].w = M.qweight[(size_t)o * C + c];
+                cur[q][r].s = M.scales[(size_t)o * groups + g];
+            }
         }
     }
 
-    // stage x (already in g_index order) into padded chunks
-    {
-        const float4 *xin = reinterpret_cast<const float4 *>(M.x + (size_t)b * in);
-        for (int j4 = tid; j4 < (in >> 2); j4 += NW * 64) {
-            const float4 v = xin[j4];
-            const int j = j4 << 2;
-            *reinterpret_cast<float4 *>(&xs[(j >> 5) * kChunkPad + (j & 31)]) = v;
-        }
-    }
-    __syncthreads();
-    for (int cc = tid; cc < C; cc += NW * 64) {
-        const float4 *p = reinterpret_cast<const float4 *>(&xs[cc * kChunkPad]);
-        float s = 0.f;
+    float ssq = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float4 v = p[i];
-            s += (v.x + v.y) + (v.z + v.w);
-        }
-        xsum[cc] = s;
+    for (int q = 0; q < NM; q++) {
+        const Q4Mat &M = L.m[mi + q];
+        const float part = stage_input<NW>(M.x + (size_t)b * in, M.wn, in, lds + q * xstride,
+                                           lds + q * xstride + C * kChunkPad, tid);
+        if (q == 0) ssq = part;
+    }
+    const bool norm = L.m[mi].wn != nullptr;
+    if (norm) {
+        ssq = wave_sum(ssq);
+        if (lane == 0) red[wave] = ssq;
     }
     __syncthreads();
     if (!active) return;
-
-    float acc[R];
+    float ss = 1.0f;
+    if (norm) { // rmsnorm scale, src/models.rs:55-60
+        float t = 0.f;
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.f;
+        for (int i = 0; i < NW; i++) t += red[i];
+        t /= (float)in;
+        t += L.eps;
+        ss = 1.0f / sqrtf(t);
+    }
+
+    float acc[NM][R];
+#pragma unroll
+    for (int q = 0; q < NM; q++)
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[q][r] = 0.f;
 
     while (c < C) {
         // request the next chunk's weights before computing on this one
         const int cn = c + 64;
-        uint4 wnext[R];
-        float snext[R];
-        int32_t znext = 0;
+        RowLoad nxt[NM][R];
+        int32_t znext[NM];
+#pragma unroll
+        for (int q = 0; q < NM; q++) znext[q] = 0;
         if (cn < C) {
             const int g = cn / CPG;
-            znext = M.qzeros[(size_t)(o0 >> 3) * groups + g];
+#pragma unroll
+            for (int q = 0; q < NM; q++) {
+                const Q4Mat &M = L.m[mi + q];
+                znext[q] = M.qzeros[(size_t)(o0 >> 3) * groups + g];
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int o = min(o0 + r, n_out - 1);
+                    nxt[q][r].w = M.qweight[(size_t)o * C + cn];
+                    nxt[q][r].s = M.scales[(size_t)o * groups + g];
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            const float *xs = lds + q * xstride;
+            float x[32];
+            {
+                const float4 *p = reinterpret_cast<const float4 *>(&xs[c * kChunkPad]);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4 v = p[i];
+                    x[4 * i + 0] = v.x;
+                    x[4 * i + 1] = v.y;
+                    x[4 * i + 2] = v.z;
+                    x[4 * i + 3] = v.w;
+                }
+            }
+            const float sx = xs[C * kChunkPad + c];
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const int o = min(o0 + r, M.out - 1);
-                wnext[r] = M.qweight[(size_t)o * C + cn];
-                snext[r] = M.scales[(size_t)o * groups + g];
+                const float p = chunk_dot(cur[q][r].w, x);
+                const int zn = (zcur[q] >> (4 * ((o0 + r) & 7))) & 15;
+                const float z1 = (float)(zn + 1);
+                const float t = fmaf(p, 512.0f, -z1 * sx);
+                acc[q][r] = fmaf(cur[q][r].s, t, acc[q][r]);
             }
         }
-        float x[32];
-        {
-            const float4 *p = reinterpret_cast<const float4 *>(&xs[c * kChunkPad]);
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float4 v = p[i];
-                x[4 * i + 0] = v.x;
-                x[4 * i + 1] = v.y;
-                x[4 * i + 2] = v.z;
-                x[4 * i + 3] = v.w;
-            }
-        }
-        const float sx = xsum[c];
+        for (int q = 0; q < NM; q++) {
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            float lo = 0.f, hi = 0.f;
-            chunk_dot(wcur[r], x, lo, hi);
-            const int zn = (zcur >> (4 * ((o0 + r) & 7))) & 15;
-            const float z1 = (float)(zn + 1);
-            float t = fmaf(hi, 0.0625f, lo);
-            t = fmaf(-z1, sx, t);
-            acc[r] = fmaf(scur[r], t, acc[r]);
+            for (int r = 0; r < R; r++) cur[q][r] = nxt[q][r];
+            zcur[q] = znext[q];
         }
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            wcur[r] = wnext[r];
-            scur[r] = snext[r];
-        }
-        zcur = znext;
         c = cn;
     }
 
+    // wave reduction, then lane r finishes row o0 + r
+    float mine[NM];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        const float v = wave_sum(acc[r]);
-        const int o = o0 + r;
-        if (lane == 0 && o < M.out) {
-            float out = v;
-            if (L.epi == Q4_EPI_RESIDUAL) out = M.res[(size_t)b * M.y_stride + o] + v;
-            const int dst = M.scatter ? M.scatter[o] : o;
-            M.y[(size_t)b * M.y_stride + dst] = out;
+    for (int q = 0; q < NM; q++) mine[q] = 0.f;
+#pragma unroll
+    for (int q = 0; q < NM; q++)
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float v = wave_sum(acc[q][r]);
+            if (lane == r) mine[q] = v;
         }
+    const int o = o0 + lane;
+    if (lane < R && o < n_out) {
+        const Q4Epi &E = L.e;
+        const size_t row = (size_t)b * n_out;
+        float v = mine[0] * ss;
+        if (PAIR) { // silu(w1 x) * (w3 x), src/models.rs:92-98
+            const float u = mine[NM - 1] * ss;
+            v = v * (1.0f / (1.0f + expf(-v)));
+            v = v * u;
+        } else if (E.kind == Q4_EPI_RESIDUAL) {
+            v = E.res[row + o] + v;
+        }
+        if (E.kind != Q4_EPI_SCATTER_ONLY) L.m[mi].y[row + o] = v;
+        for (int t = 0; t < E.n_scatter; t++) E.sc_out[t][row + E.sc_idx[t][o]] = v;
     }
 }
 
-template <int G, int R, int NW>
+template <int G, int R, int NW, bool PAIR>
 int launch_t(Q4Launch &L, hipStream_t stream) {
     int total = 0;
     for (int i = 0; i < L.n_mats; i++) {
         L.m[i].row_blocks = (L.m[i].out + NW * R - 1) / (NW * R);
         total += L.m[i].row_blocks;
     }
+    if (PAIR) total = L.m[0].row_blocks;
     const int C = L.in / 32;
-    const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float);
-    auto kern = q4_matvec_kernel<G, R, NW>;
+    const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
+    auto kern = q4_matvec_kernel<G, R, NW, PAIR>;
+    if (lds + 256 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
     if (lds > 64 * 1024) {
-        static bool raised = false; // per instantiation
-        if (!raised) {
+        static size_t raised = 0; // per instantiation: the largest dynamic LDS size allowed so far
+        if (lds > raised) {
             L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            raised = true;
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            raised = lds;
         }
     }
-    if (lds > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
     dim3 grid(total, L.batch), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, stream, L);
     L2_HIP(hipGetLastError());
@@ -222,12 +332,16 @@ int launch_t(Q4Launch &L, hipStream_t stream) {
 template <int G>
 int launch_g(Q4Launch &L, hipStream_t stream, int R, int NW) {
 #define Q4_CASE(r, nw) \
-    if (R == r && NW == nw) return launch_t<G, r, nw>(L, stream);
+    if (!L.pair && R == r && NW == nw) return launch_t<G, r, nw, false>(L, stream);
+#define Q4_PAIR(r, nw) \
+    if (L.pair && R == r && NW == nw) return launch_t<G, r, nw, true>(L, stream);
     Q4_CASE(2, 4) Q4_CASE(4, 4) Q4_CASE(8, 4)
     Q4_CASE(2, 8) Q4_CASE(4, 8) Q4_CASE(8, 8)
-    Q4_CASE(2, 16) Q4_CASE(4, 16) Q4_CASE(8, 16)
+    Q4_CASE(2, 16) Q4_CASE(4, 16)
+    Q4_PAIR(2, 4) Q4_PAIR(4, 4) Q4_PAIR(2, 8) Q4_PAIR(4, 8) Q4_PAIR(2, 16)
 #undef Q4_CASE
-    return l2_fail(L2_ERR_ARG, "q4 matvec: no kernel for R=%d NW=%d", R, NW);
+#undef Q4_PAIR
+    return l2_fail(L2_ERR_ARG, "q4 matvec: no kernel for R=%d NW=%d pair=%d", R, NW, L.pair);
 }
 
 int env_int(const char *name, int dflt) {
@@ -243,6 +357,9 @@ int q4_matvec_launch(Q4Launch &L, hipStream_t stream) {
         return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d must be a multiple of 32 and of the group size %d",
                        L.in, L.group_size);
     if (L.batch < 1 || L.batch > 65535) return l2_fail(L2_ERR_RANGE, "q4 matvec: batch=%d", L.batch);
+    if (L.e.n_scatter < 0 || L.e.n_scatter > 3) return l2_fail(L2_ERR_ARG, "q4 matvec: %d scatter targets", L.e.n_scatter);
+    if (L.pair && (L.n_mats != 2 || L.m[0].out != L.m[1].out))
+        return l2_fail(L2_ERR_ARG, "q4 matvec: a pair launch takes two matrices of equal height");
     long rows = 0;
     for (int i = 0; i < L.n_mats; i++) {
         if (L.m[i].out % 8 != 0) return l2_fail(L2_ERR_ARG, "q4 matvec: out=%d not a multiple of 8", L.m[i].out);
@@ -253,14 +370,17 @@ int q4_matvec_launch(Q4Launch &L, hipStream_t stream) {
     static const int forced_r = env_int("L2_Q4_R", 0);
     static const int forced_nw = env_int("L2_Q4_NW", 0);
     const int C = L.in / 32;
-    int R = rows >= 32768 ? 8 : rows >= 8192 ? 4 : 2;
+    int R = rows >= 32768 ? 4 : 2;
+    if (L.pair) R = 2;
     // Waves per block: big inputs need most of a CU's LDS for x, so one block
     // must bring enough waves by itself.
-    const size_t lds = (size_t)(C * kChunkPad + C) * 4;
+    const size_t lds = (size_t)(C * kChunkPad + C) * 4 * (L.pair ? 2 : 1);
     int NW = lds > 80 * 1024 ? 16 : lds > 40 * 1024 ? 8 : 4;
     if (forced_r) R = forced_r;
     if (forced_nw) NW = forced_nw;
     if (NW == 16 && R > 4) R = 4; // 1024-thread blocks leave 128 VGPRs per lane
+    if (L.pair && R > 4) R = 4;
+    if (L.pair && NW == 16) R = 2;
     switch (L.group_size) {
         case 32: return launch_g<32>(L, stream, R, NW);
         case 64: return launch_g<64>(L, stream, R, NW);

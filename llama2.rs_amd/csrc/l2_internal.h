@@ -44,33 +44,45 @@ struct DevQLinear {
 
 // ---- q4 matvec launch description ------------------------------------------
 
-enum { Q4_EPI_STORE = 0, Q4_EPI_RESIDUAL = 1 };
+enum {
+    Q4_EPI_STORE = 0,       // y[b][o] = v (+ scatter targets)
+    Q4_EPI_RESIDUAL = 1,    // v += res[b][o]; y[b][o] = v (+ scatter targets)
+    Q4_EPI_SCATTER_ONLY = 2 // scatter targets only
+};
 
 struct Q4Mat {
     const uint4 *qweight;
     const int32_t *qzeros;
     const float *scales;
-    const float *x;         // input already in this layer's g_index order: [B][in]
-    float *y;               // [B][y_stride]
-    const float *res;       // Q4_EPI_RESIDUAL: y = res + W x   (may alias y)
-    const int32_t *scatter; // optional: write y[b][scatter[o]] instead of y[b][o]
+    const float *x;  // input already in this layer's g_index order: [B][in]
+    const float *wn; // rmsnorm weights in the same order, or null: x is used as it is
+    float *y;        // [B][out]
     int out;
-    int y_stride;
-    int row_blocks;         // blocks of grid.x that belong to this matrix
+    int row_blocks;  // blocks of grid.x that belong to this matrix
+};
+
+struct Q4Epi {
+    int kind;
+    const float *res;          // Q4_EPI_RESIDUAL: [B][out] (may alias y)
+    int n_scatter;             // 0..3
+    const int32_t *sc_idx[3];  // inverse act-order permutation of a following layer
+    float *sc_out[3];          // [B][out]: sc_out[t][b][sc_idx[t][o]] = v
 };
 
 struct Q4Launch {
     Q4Mat m[3];
+    Q4Epi e;
     int n_mats;
     int in;      // shared by all matrices of one launch
     int groups;
     int group_size;
-    int epi;
     int batch;
+    int pair;    // 1: m[0], m[1] are w1, w3; v = silu(m0 row) * (m1 row)
+    float eps;   // rmsnorm epsilon, used when wn is set
 };
 
-// Launch the B=1-per-column fp32 dequant matvec for up to 3 matrices that share
-// `in` (e.g. wq|wk|wv or w1|w3).  Fills row_blocks itself.
+// Launch the fp32 dequant matvec for up to 3 matrices that share `in`
+// (wq|wk|wv), or a (w1, w3) pair.  Fills row_blocks itself.
 int q4_matvec_launch(Q4Launch &L, hipStream_t stream);
 
 // ---- the other per-token kernels -------------------------------------------
@@ -81,25 +93,40 @@ struct ScatterTargets {
     int n;
 };
 
-int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int vocab, int B,
-                 hipStream_t st);
-// out_c[b][inv_c[i]] = (w[i] * ss_b) * x[b][i]; inv == nullptr writes in place order.
-int rmsnorm_scatter_launch(const float *x, const float *w, float eps, int dim, int B,
-                           const ScatterTargets &t, hipStream_t st);
+// x[b] = emb[tokens[b]], also delivered through t; clears the running argmax.
+int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int B, const ScatterTargets &t,
+                 unsigned long long *amax_key, hipStream_t st);
 int gather_launch(float *out, const float *x, const int32_t *g_index, int n, int B, hipStream_t st);
 int rope_kv_launch(float *q, const float *k, const float *v, const int32_t *pos, const float *cos_t,
                    const float *sin_t, float *kcache_l, float *vcache_l, int n_heads, int n_kv_heads,
                    int head_size, int B, hipStream_t st);
-// out[b][scatter[i]] (or out[b][i]) = attention for query b at position pos[b].
+// Batched attention over an already written cache: out[b][scatter[i]] for query b at pos[b].
 int attention_launch(float *out, const float *q, const float *kcache_l, const float *vcache_l,
                      const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
                      int head_size, int max_pos, int B, hipStream_t st);
-int silu_scatter_launch(float *out, const float *a, const float *b, const int32_t *scatter, int n,
-                        int B, hipStream_t st);
-// y[o] = sum_i w[o][i] x[i]; if amax_key != nullptr also folds (value,index) into it.
-int dense_matvec_launch(float *y, const float *w, const float *x, int in, int out,
+
+// Decode attention (one query) with RoPE and the cache write folded in.
+struct AttnDecode {
+    const float *q;      // [dim]    raw query of this step
+    const float *k_new;  // [kv_dim] raw key
+    const float *v_new;  // [kv_dim] value
+    float *kcache, *vcache;          // this layer: [max_seq][kv_dim]
+    const float *cos_t, *sin_t;      // [max_seq][head_size/2]
+    const int32_t *dpos;             // device: position of this step
+    float *out;                      // [dim], written through scatter
+    const int32_t *scatter;
+    float *part;                     // split workspace: [n_heads][max_splits][130]
+    int n_heads, n_kv_heads;
+    int ts;                          // timesteps per split (multiple of 64)
+    int n_splits;                    // grid.y; 1 = no combine pass
+    int max_splits;
+};
+int attention_decode_launch(const AttnDecode &a, hipStream_t st);
+
+// logits = wcls (rmsnorm(x, wn)); folds (value, index) into amax_key when set.
+// wn == nullptr: plain Linear::matvec of x.
+int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
                         unsigned long long *amax_key, hipStream_t st);
-int fill_u64_launch(unsigned long long *p, unsigned long long v, int n, hipStream_t st);
 // pos = dpos[0]; next = pos < n_prompt ? prompt[pos] : index(amax_key);
 // out_ids[pos - pos0] = next; tok[0] = next; dpos[0] = pos + 1.
 int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,

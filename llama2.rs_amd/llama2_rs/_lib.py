@@ -10,7 +10,8 @@ import ctypes as C
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_PKG), "libllama2_hip.so")
+# LLAMA2_HIP_LIB names another build of the same library (e.g. an instrumented one).
+LIB_PATH = os.environ.get("LLAMA2_HIP_LIB") or os.path.join(os.path.dirname(_PKG), "libllama2_hip.so")
 
 L2_OK = 0
 ERR_NAMES = {-1: "L2_ERR_ARG", -2: "L2_ERR_IO", -3: "L2_ERR_FORMAT", -4: "L2_ERR_HIP", -5: "L2_ERR_RANGE"}
@@ -70,6 +71,9 @@ SIGNATURES = {
     "l2_generate_greedy": (_I, [_VP, _VP, _VP, _I, _I, _I, _VP, C.POINTER(_I), C.POINTER(C.c_double)]),
     "l2_qlinear_bench": (_I, [C.POINTER(_VP), _I, _I, C.POINTER(C.c_float)]),
     "l2_decode_bench": (_I, [_VP, _VP, C.c_int32, C.c_int32, _I, _VP, C.POINTER(C.c_float)]),
+    "l2_kernel_class_count": (_I, []),
+    "l2_kernel_class_name": (C.c_char_p, [_I]),
+    "l2_decode_profile": (_I, [_VP, _VP, C.c_int32, C.c_int32, _I, _VP, _VP]),
     "l2_copy_bench": (_I, [_SZ, _I, C.POINTER(C.c_float)]),
 }
 

@@ -190,6 +190,14 @@ class Model:
         check(lib().l2_decode_bench(self.h, self.state, token, pos, n_tokens, _p(out), C.byref(ms)))
         return out, ms.value
 
+    def decode_profile(self, token: int, pos: int, n_tokens: int):
+        """{class name: (ms summed over the run, launches)} from per-launch HIP events."""
+        n = lib().l2_kernel_class_count()
+        ms = np.zeros(n, np.float32)
+        cnt = np.zeros(n, np.int32)
+        check(lib().l2_decode_profile(self.h, self.state, token, pos, n_tokens, _p(ms), _p(cnt)))
+        return {lib().l2_kernel_class_name(i).decode(): (float(ms[i]), int(cnt[i])) for i in range(n)}
+
     def read_kv(self, layer: int, pos0: int, npos: int):
         d = self.dims
         k = np.empty((npos, d.n_kv_heads, d.head_size), np.float32)
