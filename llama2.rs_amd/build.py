@@ -24,6 +24,7 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", f"--off
 SOURCES = {
     # file: extra flags
     "kernels_q4.hip": [],
+    "kernels_q4_stream.hip": [],
     # the block kernels keep the reference's rounded-multiply-then-add where they restate it
     "kernels_misc.hip": ["-ffp-contract=off"],
     "host.cpp": ["-x", "hip", "-ffp-contract=off"],

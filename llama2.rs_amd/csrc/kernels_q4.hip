@@ -31,108 +31,13 @@
 // also delivers the new residual stream in the input order of up to three
 // following layers; SiLU gate over a (w1, w3) pair of rows
 // (src/models.rs:271-276) delivered in w2's input order.
-#include "l2_internal.h"
+#include <string.h>
+
+#include "q4_common.h"
 
 namespace {
 
-constexpr int kChunkPad = 36; // floats per staged chunk of 32
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_xchg(float v) {
-    int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
-    return __builtin_bit_cast(float, r);
-}
-
-// Sum over the 64 lanes of a wave; every lane gets the result.
-__device__ __forceinline__ float wave_sum(float v) {
-    v += dpp_xchg<0xB1>(v);  // quad_perm [1,0,3,2]
-    v += dpp_xchg<0x4E>(v);  // quad_perm [2,3,0,1]
-    v += dpp_xchg<0x141>(v); // row_half_mirror
-    v += dpp_xchg<0x140>(v); // row_mirror
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
-}
-
-typedef float v2f __attribute__((ext_vector_type(2)));
-
-// 32 nibbles of one row against 32 inputs: returns 2^-9 * sum_k n_k x_k.
-//
-// A nibble n parked in the low half of a byte, 0000nnnn, read as an OCP FP8
-// E4M3 number is exactly n * 2^-9 (subnormal for n < 8, exponent 1 above, the
-// same step on both sides), so v_cvt_pk_f32_fp8 turns two nibbles into two
-// floats in one instruction.  Even nibbles come from w & 0x0F0F0F0F, odd ones
-// from (w >> 4) & 0x0F0F0F0F.  The power of two is undone exactly by the
-// caller.
-__device__ __forceinline__ float chunk_dot(const uint4 w, const float (&x)[32]) {
-    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
-    float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        const uint32_t l = words[d] & 0x0F0F0F0Fu;
-        const uint32_t h = (words[d] >> 4) & 0x0F0F0F0Fu;
-        const v2f l01 = __builtin_amdgcn_cvt_pk_f32_fp8(l, false); // nibbles 0, 2
-        const v2f l23 = __builtin_amdgcn_cvt_pk_f32_fp8(l, true);  // nibbles 4, 6
-        const v2f h01 = __builtin_amdgcn_cvt_pk_f32_fp8(h, false); // nibbles 1, 3
-        const v2f h23 = __builtin_amdgcn_cvt_pk_f32_fp8(h, true);  // nibbles 5, 7
-        a0 = fmaf(l01.x, x[8 * d + 0], a0);
-        a1 = fmaf(h01.x, x[8 * d + 1], a1);
-        a0 = fmaf(l01.y, x[8 * d + 2], a0);
-        a1 = fmaf(h01.y, x[8 * d + 3], a1);
-        a0 = fmaf(l23.x, x[8 * d + 4], a0);
-        a1 = fmaf(h23.x, x[8 * d + 5], a1);
-        a0 = fmaf(l23.y, x[8 * d + 6], a0);
-        a1 = fmaf(h23.y, x[8 * d + 7], a1);
-    }
-    return a0 + a1;
-}
-
-// Stage one input vector into padded chunks + chunk sums; returns this
-// thread's share of sum(x^2) (of the raw input, before the norm weight).
-template <int NW>
-__device__ __forceinline__ float stage_input(const float *__restrict__ xin_f, const float *__restrict__ wn_f,
-                                             int in, float *xs, float *xsum, int tid) {
-    const float4 *xin = reinterpret_cast<const float4 *>(xin_f);
-    const float4 *wn = reinterpret_cast<const float4 *>(wn_f);
-    const int n4 = in >> 2;
-    constexpr int T = NW * 64, U = 4;
-    float ssq = 0.f;
-    for (int base = 0; base < n4; base += T * U) {
-        float4 v[U], g[U];
-        // all loads of a batch are issued before the first one is consumed
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int j4 = base + u * T + tid;
-            v[u] = j4 < n4 ? xin[j4] : make_float4(0.f, 0.f, 0.f, 0.f);
-            g[u] = (wn_f && j4 < n4) ? wn[j4] : make_float4(1.f, 1.f, 1.f, 1.f);
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int j4 = base + u * T + tid;
-            if (wn_f) {
-                ssq = fmaf(v[u].x, v[u].x, ssq);
-                ssq = fmaf(v[u].y, v[u].y, ssq);
-                ssq = fmaf(v[u].z, v[u].z, ssq);
-                ssq = fmaf(v[u].w, v[u].w, ssq);
-                v[u].x *= g[u].x;
-                v[u].y *= g[u].y;
-                v[u].z *= g[u].z;
-                v[u].w *= g[u].w;
-            }
-            // the 8 consecutive lanes that hold one chunk add up its sum
-            float s = (v[u].x + v[u].y) + (v[u].z + v[u].w);
-            s += dpp_xchg<0xB1>(s);  // lanes ^1
-            s += dpp_xchg<0x4E>(s);  // lanes ^2
-            s += dpp_xchg<0x141>(s); // 7 - lane within each 8: the other quad
-            if (j4 < n4) {
-                const int j = j4 << 2;
-                *reinterpret_cast<float4 *>(&xs[(j >> 5) * kChunkPad + (j & 31)]) = v[u];
-                if ((tid & 7) == 0) xsum[j >> 5] = s;
-            }
-        }
-    }
-    return ssq;
-}
+using namespace q4;
 
 struct RowLoad {
     uint4 w;
@@ -365,6 +270,12 @@ int q4_matvec_launch(Q4Launch &L, hipStream_t stream) {
         if (L.m[i].out % 8 != 0) return l2_fail(L2_ERR_ARG, "q4 matvec: out=%d not a multiple of 8", L.m[i].out);
         rows += L.m[i].out;
     }
+    // The row-streaming form is the default; L2_Q4_IMPL=tile selects the row-tile form.
+    static const int impl_tile = []() {
+        const char *v = getenv("L2_Q4_IMPL");
+        return (v && !strcmp(v, "tile")) ? 1 : 0;
+    }();
+    if (!impl_tile && q4_stream_supports(L)) return q4_stream_launch(L, stream);
     // Rows per wave: enough waves to cover 256 CUs several times over, more
     // rows per wave (less LDS traffic per weight byte) once there are plenty.
     static const int forced_r = env_int("L2_Q4_R", 0);

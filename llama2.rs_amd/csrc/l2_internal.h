@@ -79,11 +79,15 @@ struct Q4Launch {
     int batch;
     int pair;    // 1: m[0], m[1] are w1, w3; v = silu(m0 row) * (m1 row)
     float eps;   // rmsnorm epsilon, used when wn is set
+    int rows_per_block; // filled by the streaming launcher
 };
 
 // Launch the fp32 dequant matvec for up to 3 matrices that share `in`
 // (wq|wk|wv), or a (w1, w3) pair.  Fills row_blocks itself.
 int q4_matvec_launch(Q4Launch &L, hipStream_t stream);
+// The two forms of the kernel behind q4_matvec_launch.
+int q4_stream_launch(Q4Launch &L, hipStream_t stream);
+bool q4_stream_supports(const Q4Launch &L);
 
 // ---- the other per-token kernels -------------------------------------------
 
