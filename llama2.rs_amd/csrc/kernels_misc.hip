@@ -69,14 +69,15 @@ __device__ __forceinline__ float block_max(float v, float *red) {
 // forward pass, so it also clears the running argmax.
 __global__ void embed_kernel(float *x, const float *emb, const int32_t *tokens, int dim, ScatterTargets t,
                              unsigned long long *amax) {
-    const int b = blockIdx.x;
+    const int b = blockIdx.y;
     const float *src = emb + (size_t)tokens[b] * dim;
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < dim) {
         const float v = src[i];
         x[(size_t)b * dim + i] = v;
         for (int c = 0; c < t.n; c++) t.out[c][(size_t)b * dim + t.inv[c][i]] = v;
     }
-    if (amax && b == 0 && threadIdx.x == 0) amax[0] = 0ull;
+    if (amax && b == 0 && i == 0) amax[0] = 0ull;
 }
 
 // out[b][j] = x[b][g_index[j]]  (src/gptq.rs:110-114), for callers that hand the
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     __shared__ float qs[QG * HS];
     __shared__ float knew[HS];
     __shared__ float ml[QG][2];
-    __shared__ float half2[QG][HS];
+    __shared__ float vred[7][HS];
     const int kvh = blockIdx.x, sp = blockIdx.y;
     const int pos = A.dpos[0];
     const int t0 = sp * A.ts;
@@ -305,36 +306,54 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     }
     __syncthreads();
 
-    // weighted values: thread -> (dim d, parity of t)
-    const int d = tid & (HS - 1), par = tid >> 7;
-    float acc[QG];
+    // weighted values: thread -> (4 dims, one of 8 interleaved sets of timesteps)
+    const int d4 = tid & 31, tg = tid >> 5;
+    float4 acc[QG];
 #pragma unroll
-    for (int j = 0; j < QG; j++) acc[j] = 0.f;
-    const float *vbase = A.vcache + (size_t)kvh * HS + d;
-#pragma unroll 4
-    for (int tt = par; tt < n; tt += 2) {
+    for (int j = 0; j < QG; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float *vbase = A.vcache + (size_t)kvh * HS + d4 * 4;
+#pragma unroll 2
+    for (int tt = tg; tt < n; tt += 8) {
         const int t = t0 + tt;
-        const float v = (t == pos) ? A.v_new[(size_t)kvh * HS + d] : vbase[(size_t)t * kv_dim];
-#pragma unroll
-        for (int j = 0; j < QG; j++) acc[j] = fmaf(sc[j * A.ts + tt], v, acc[j]);
-    }
-    if (par == 1) {
-#pragma unroll
-        for (int j = 0; j < QG; j++) half2[j][d] = acc[j];
-    }
-    __syncthreads();
-    if (par == 0) {
+        const float4 v = (t == pos) ? *reinterpret_cast<const float4 *>(A.v_new + (size_t)kvh * HS + d4 * 4)
+                                    : *reinterpret_cast<const float4 *>(vbase + (size_t)t * kv_dim);
 #pragma unroll
         for (int j = 0; j < QG; j++) {
-            const float o = acc[j] + half2[j][d];
+            const float p = sc[j * A.ts + tt];
+            acc[j].x = fmaf(p, v.x, acc[j].x);
+            acc[j].y = fmaf(p, v.y, acc[j].y);
+            acc[j].z = fmaf(p, v.z, acc[j].z);
+            acc[j].w = fmaf(p, v.w, acc[j].w);
+        }
+    }
+    // fold the 8 sets: sets 1..7 park their sums, set 0 adds them in order
+#pragma unroll
+    for (int j = 0; j < QG; j++) {
+        __syncthreads();
+        if (tg > 0) *reinterpret_cast<float4 *>(&vred[tg - 1][d4 * 4]) = acc[j];
+        __syncthreads();
+        if (tg == 0) {
+            float4 o = acc[j];
+#pragma unroll
+            for (int k = 0; k < 7; k++) {
+                const float4 e = *reinterpret_cast<const float4 *>(&vred[k][d4 * 4]);
+                o.x += e.x;
+                o.y += e.y;
+                o.z += e.z;
+                o.w += e.w;
+            }
             const int h = kvh * QG + j;
+            const float vals[4] = {o.x, o.y, o.z, o.w};
             if (A.n_splits == 1) {
-                const int i = h * HS + d;
-                A.out[A.scatter ? A.scatter[i] : i] = o / ml[j][1];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int i = h * HS + d4 * 4 + e;
+                    A.out[A.scatter ? A.scatter[i] : i] = vals[e] / ml[j][1];
+                }
             } else {
                 float *p = A.part + ((size_t)h * A.max_splits + sp) * (HS + 2);
-                p[d] = o;
-                if (d == 0) {
+                *reinterpret_cast<float4 *>(p + d4 * 4) = o;
+                if (d4 == 0) {
                     p[HS] = ml[j][0];
                     p[HS + 1] = ml[j][1];
                 }
@@ -408,36 +427,49 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float
     __syncthreads();
     const int n4 = in / 4;
     const int waves_total = gridDim.x * 4;
-    for (int o = (blockIdx.x * 4 + wave) * 2; o < out; o += waves_total * 2) {
-        const int o1 = min(o + 1, out - 1);
-        const float4 *r0 = reinterpret_cast<const float4 *>(w + (size_t)o * in);
-        const float4 *r1 = reinterpret_cast<const float4 *>(w + (size_t)o1 * in);
-        float a0 = 0.f, a1 = 0.f;
-#pragma unroll 4
-        for (int j = lane; j < n4; j += 64) {
-            const float4 xv = reinterpret_cast<const float4 *>(xs)[j];
-            const float4 w0 = r0[j], w1 = r1[j];
-            a0 = fmaf(w0.x, xv.x, a0);
-            a0 = fmaf(w0.y, xv.y, a0);
-            a0 = fmaf(w0.z, xv.z, a0);
-            a0 = fmaf(w0.w, xv.w, a0);
-            a1 = fmaf(w1.x, xv.x, a1);
-            a1 = fmaf(w1.y, xv.y, a1);
-            a1 = fmaf(w1.z, xv.z, a1);
-            a1 = fmaf(w1.w, xv.w, a1);
+    constexpr int RW = 4; // rows per wave and pass: RW x 2 loads of 16 bytes in flight per lane
+    for (int o = (blockIdx.x * 4 + wave) * RW; o < out; o += waves_total * RW) {
+        const float4 *r[RW];
+        float a[RW];
+#pragma unroll
+        for (int k = 0; k < RW; k++) {
+            r[k] = reinterpret_cast<const float4 *>(w + (size_t)min(o + k, out - 1) * in);
+            a[k] = 0.f;
         }
-        a0 = wave_sum(a0) * ss;
-        a1 = wave_sum(a1) * ss;
-        if (lane == 0) {
-            y[o] = a0;
-            unsigned long long key = amax_key(a0, o);
-            if (o + 1 < out) {
-                y[o + 1] = a1;
-                const unsigned long long k1 = amax_key(a1, o + 1);
-                key = k1 > key ? k1 : key;
+        for (int j = lane; j < n4; j += 128) {
+            const int j2 = j + 64;
+            const bool two = j2 < n4;
+            float4 wv[RW][2];
+#pragma unroll
+            for (int k = 0; k < RW; k++) {
+                wv[k][0] = r[k][j];
+                wv[k][1] = two ? r[k][j2] : make_float4(0.f, 0.f, 0.f, 0.f);
             }
-            if (amax) atomicMax(amax, key);
+            const float4 x0 = reinterpret_cast<const float4 *>(xs)[j];
+            const float4 x1 = two ? reinterpret_cast<const float4 *>(xs)[j2] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int k = 0; k < RW; k++) {
+                a[k] = fmaf(wv[k][0].x, x0.x, a[k]);
+                a[k] = fmaf(wv[k][0].y, x0.y, a[k]);
+                a[k] = fmaf(wv[k][0].z, x0.z, a[k]);
+                a[k] = fmaf(wv[k][0].w, x0.w, a[k]);
+                a[k] = fmaf(wv[k][1].x, x1.x, a[k]);
+                a[k] = fmaf(wv[k][1].y, x1.y, a[k]);
+                a[k] = fmaf(wv[k][1].z, x1.z, a[k]);
+                a[k] = fmaf(wv[k][1].w, x1.w, a[k]);
+            }
         }
+        unsigned long long key = 0ull;
+#pragma unroll
+        for (int k = 0; k < RW; k++) {
+            const float v = wave_sum(a[k]) * ss;
+            if (lane == 0 && o + k < out) {
+                y[o + k] = v;
+                const unsigned long long kk = amax_key(v, o + k);
+                key = kk > key ? kk : key;
+            }
+        }
+        if (lane == 0 && amax) atomicMax(amax, key);
     }
 }
 
@@ -477,7 +509,7 @@ __global__ void fill_pattern_kernel(float *p, size_t n, uint64_t seed) {
 int embed_launch(float *x, const float *emb, const int32_t *tokens, int dim, int B, const ScatterTargets &t,
                  unsigned long long *amax_key, hipStream_t st) {
     if (t.n < 0 || t.n > 3) return l2_fail(L2_ERR_ARG, "embed: %d targets", t.n);
-    hipLaunchKernelGGL(embed_kernel, dim3(B), dim3(1024), 0, st, x, emb, tokens, dim, t, amax_key);
+    hipLaunchKernelGGL(embed_kernel, dim3((dim + 255) / 256, B), dim3(256), 0, st, x, emb, tokens, dim, t, amax_key);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }
@@ -534,7 +566,7 @@ int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
 int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
                         unsigned long long *amax_key, hipStream_t st) {
     if (in % 4 || in * 4 > 64 * 1024) return l2_fail(L2_ERR_ARG, "dense matvec: in=%d", in);
-    int blocks = (out + 7) / 8;
+    int blocks = (out + 15) / 16;
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL(dense_matvec_kernel, dim3(blocks), dim3(256), (size_t)in * 4, st, y, w, x, wn, eps, in,
                        out, amax_key);

@@ -30,7 +30,10 @@ template <int G, int NWK, int S, bool PAIR>
 __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L) {
     constexpr int NM = PAIR ? 2 : 1;
     constexpr int NW = NWK * S;
-    constexpr int P = PAIR ? 2 : 4; // rows (row pairs) in flight per stream
+#ifndef Q4S_P
+#define Q4S_P 4
+#endif
+    constexpr int P = PAIR ? Q4S_P / 2 : Q4S_P; // rows (row pairs) in flight per stream
     constexpr int TR = P * S;       // rows per reduction tile
     constexpr int PW = NWK * 4;     // partials per row
     constexpr int CPG = G / 32;     // chunks per group
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
                 const Q4Mat &M = L.m[mi + q];
                 d[q].w = M.qweight[(size_t)o * C + c];
 #ifdef L2_Q4_DEBUG
-                if (L.e.kind == 103) { // weights only
+                if (L.e.kind >= 103) { // weights only
                     d[q].s = 1.f;
                     d[q].z = 0;
                     continue;
@@ -174,6 +177,9 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
                 if ((lane & 15) == 0) part[buf][u * S + stream][q][kslice * 4 + (lane >> 4)] = v;
             }
         }
+#ifdef L2_Q4_DEBUG
+        if (L.e.kind == 104) continue; // no reduction barrier, no epilogue
+#endif
         __syncthreads();
         if (tid < TR) {
             const int o = row0 + tile * TR + tid;
@@ -219,7 +225,7 @@ int cu_count() {
 template <int G, int NWK, int S, bool PAIR>
 int launch_s(Q4Launch &L, hipStream_t stream) {
     constexpr int NW = NWK * S;
-    constexpr int TR = (PAIR ? 2 : 4) * S;
+    constexpr int TR = (PAIR ? Q4S_P / 2 : Q4S_P) * S;
     const int C = L.in / 32;
     const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
     if (lds + 8 * 1024 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
