@@ -179,6 +179,43 @@ int l2_decode_greedy(l2_model *m, l2_state *s, int32_t token, int32_t pos, int32
 int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *prompt, int n_prompt, int steps,
                        int use_prefill, int32_t *out_ids, int *n_out, double *ms);
 
+/* ---- text surface: tokenizer, Random, generate on strings ----------------- */
+
+typedef struct l2_tokenizer l2_tokenizer; /* Tokenizer (src/tokenizer.rs:13-19) */
+typedef struct l2_random l2_random;       /* Random    (src/util.rs:55-58)      */
+
+/* Tokenizer::new (src/tokenizer.rs:41-44, load :22-37): the llama2.c format,
+ * i32 max_token_length then vocab_size x {f32 score, i32 len, bytes}.  The
+ * reference reads VOCAB_SIZE entries; pass that count. */
+int l2_tokenizer_open(const char *path, int vocab_size, l2_tokenizer **out);
+void l2_tokenizer_free(l2_tokenizer *t);
+int l2_tokenizer_vocab_size(const l2_tokenizer *t);
+/* vocab[id] (not NUL-terminated: use *len) and vocab_scores[id]. */
+int l2_tokenizer_token(const l2_tokenizer *t, int id, const char **str, int *len, float *score);
+/* Tokenizer::bpe_encode (src/tokenizer.rs:46-108) with util::str_lookup's
+ * ids-from-260-first rule (src/util.rs:29-37).  text is UTF-8; *n receives the
+ * count; ids may be NULL to ask for it.  A character missing from the
+ * vocabulary is an error (the reference's expect("not good")). */
+int l2_tokenizer_encode(const l2_tokenizer *t, const char *text, int32_t *ids, int cap, int *n);
+
+/* Random::new (src/util.rs:61-69) seeds from the wall clock in seconds
+ * (from_clock != 0); a fixed seed is offered for tests. */
+int l2_random_new(uint64_t seed, int from_clock, l2_random **out);
+void l2_random_free(l2_random *r);
+float l2_random_f32(l2_random *r);                                   /* Random::random, :79-82  */
+int l2_random_sample(l2_random *r, const float *probabilities, int n); /* Random::sample, :102-113 */
+
+/* generate() (src/inference.rs:49-193): " " + prompt.trim() is encoded, the
+ * prefill ladder and the B=1 loop run as in l2_generate_greedy; at temperature
+ * != 0 the logits come back to the host each step and are scaled, soft-maxed
+ * and sampled there as the reference does (:165-172).  `out` receives the token
+ * strings of get_token (src/util.rs:116-123) one after the other, each followed
+ * by a NUL; *n_tokens how many; *ms the elapsed wall-clock milliseconds.  With
+ * print_tokens the strings are also written to stdout. */
+int l2_generate(l2_model *m, l2_state *s, const l2_tokenizer *t, const char *prompt, int steps,
+                l2_random *rng, float temperature, int print_tokens, char *out, size_t out_cap,
+                int *n_tokens, int64_t *ms);
+
 /* ---- measurement hooks (no counterpart in the reference: it has no
  * benchmark harness beyond the tok/s line of src/main.rs:62-65) ------------ */
 

@@ -69,6 +69,17 @@ SIGNATURES = {
     "l2_forward": (_I, [_VP, _VP, _VP, _VP, _I, _VP]),
     "l2_decode_greedy": (_I, [_VP, _VP, C.c_int32, C.c_int32, C.POINTER(C.c_int32)]),
     "l2_generate_greedy": (_I, [_VP, _VP, _VP, _I, _I, _I, _VP, C.POINTER(_I), C.POINTER(C.c_double)]),
+    "l2_tokenizer_open": (_I, [C.c_char_p, _I, C.POINTER(_VP)]),
+    "l2_tokenizer_free": (None, [_VP]),
+    "l2_tokenizer_vocab_size": (_I, [_VP]),
+    "l2_tokenizer_token": (_I, [_VP, _I, C.POINTER(C.c_char_p), C.POINTER(_I), C.POINTER(C.c_float)]),
+    "l2_tokenizer_encode": (_I, [_VP, C.c_char_p, _VP, _I, C.POINTER(_I)]),
+    "l2_random_new": (_I, [C.c_uint64, _I, C.POINTER(_VP)]),
+    "l2_random_free": (None, [_VP]),
+    "l2_random_f32": (C.c_float, [_VP]),
+    "l2_random_sample": (_I, [_VP, _VP, _I]),
+    "l2_generate": (_I, [_VP, _VP, _VP, C.c_char_p, _I, _VP, C.c_float, _I, _VP, _SZ, C.POINTER(_I),
+                         C.POINTER(C.c_int64)]),
     "l2_qlinear_bench": (_I, [C.POINTER(_VP), _I, _I, C.POINTER(C.c_float)]),
     "l2_decode_bench": (_I, [_VP, _VP, C.c_int32, C.c_int32, _I, _VP, C.POINTER(C.c_float)]),
     "l2_kernel_class_count": (_I, []),
