@@ -27,6 +27,13 @@ sys.path.insert(0, os.path.join(ROOT, "llama2.rs_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
+# HBM bytes per layer moved by the four q4 launches, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (each scaled by the reading of the plain copy kernel of known size in the same run):
+# the summaries are profiles/q4_matvec_<model>_decode_hbm_counters.txt.
+MEASURED_Q4_TRAFFIC_PER_LAYER = {
+    "7B": 49111917 + 2 * 18613005 + 24759878 + 238966 + 2 * 125405 + 265887,
+}
+
 
 def q4_bytes(n_in: int, n_out: int, G: int) -> int:
     """Algorithmic bytes of one B=1 QLinear::matvec in the reference's format:
@@ -97,6 +104,12 @@ def main() -> int:
     if pos0:
         m.fill_kv_synthetic(0, pos0, seed=a.seed)
 
+    # plain device copy of known size: the box's copy bandwidth, and the known-size
+    # kernel that counter readings are scaled by
+    copy_bytes = 1 << 28
+    copy_ms = ops.copy_bench(copy_bytes, 8)
+    copy_gbs = 2 * copy_bytes * 8 / (copy_ms * 1e-3) / 1e9
+
     # warm-up: the prompt positions, forced through the B=1 loop
     tok = 1
     for i in range(W):
@@ -123,9 +136,14 @@ def main() -> int:
         tot_b = sum(cb[c] * prof[c][1] for c in q4_classes)
         tot_ms = sum(prof[c][0] for c in q4_classes)
         achieved = tot_b / (tot_ms * 1e-3) / 1e9
+        traffic = MEASURED_Q4_TRAFFIC_PER_LAYER.get(a.model)
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                    "kernel": "q4_matvec_kernel (all four launches of a layer, event-timed)",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    # mean HBM bytes per q4 launch (a layer has four), beside the algorithmic mean
+                    "traffic": round(traffic / 4) if traffic else None,
+                    "algorithmic_bytes_per_launch": round(sum(cb[c] for c in q4_classes) / 4),
+                    "kernel": "q4 matvec: the four q4 launches of a layer (q|k|v, wo, w1|w3, w2), durations from "
+                              "the dispatches' own start/stop events",
                     "per_launch": kern}
 
     result = {
@@ -152,6 +170,7 @@ def main() -> int:
         "decode_GBs": round(token_bytes(d, pos0 + W + K // 2) * tok_s / 1e9, 1),
         "decode_frac_of_hbm_peak": round(token_bytes(d, pos0 + W + K // 2) * tok_s / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": roofline,
+        "copy_GBs": round(copy_gbs, 1),
         "setup_s": {"synth": round(t_synth, 1), "upload": round(t_upload, 1)},
     }
 

@@ -24,6 +24,7 @@
 // errors
 
 static thread_local char g_err[512] = "";
+thread_local Q4ProfHook g_q4_prof;
 
 int l2_fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -299,20 +300,30 @@ static const char *const kClassNames[K_NCLASS] = {"embed", "q4_qkv", "rope_kv", 
                                                   "q4_w13", "q4_w2", "classifier", "next_token"};
 static constexpr int kMaxSplits = 64;
 
-// Time one launch with a pair of events on the launch stream (profiling runs only).
-#define LAUNCH(cls_, call)                                          \
-    do {                                                            \
-        if (m->prof_on) {                                           \
-            l2_model::ProfRec r_{cls_, nullptr, nullptr};           \
-            L2_HIP(hipEventCreate(&r_.e0));                         \
-            L2_HIP(hipEventCreate(&r_.e1));                         \
-            L2_HIP(hipEventRecord(r_.e0, m->stream));               \
-            L2_TRY(call);                                           \
-            L2_HIP(hipEventRecord(r_.e1, m->stream));               \
-            m->prof.push_back(r_);                                  \
-        } else {                                                    \
-            L2_TRY(call);                                           \
-        }                                                           \
+// Time one launch (profiling runs only).  The q4 launches hand their events to
+// the dispatch itself; the others are bracketed by event records on the stream.
+#define LAUNCH(cls_, call)                                                          \
+    do {                                                                            \
+        if (m->prof_on) {                                                           \
+            l2_model::ProfRec r_{cls_, nullptr, nullptr};                           \
+            L2_HIP(hipEventCreate(&r_.e0));                                         \
+            L2_HIP(hipEventCreate(&r_.e1));                                         \
+            const bool q4_ = (cls_) == K_Q4_QKV || (cls_) == K_Q4_WO || (cls_) == K_Q4_W13 || (cls_) == K_Q4_W2; \
+            if (q4_) {                                                              \
+                g_q4_prof.start = r_.e0;                                            \
+                g_q4_prof.stop = r_.e1;                                             \
+                g_q4_prof.armed = true;                                             \
+                L2_TRY(call);                                                       \
+                g_q4_prof.armed = false;                                            \
+            } else {                                                                \
+                L2_HIP(hipEventRecord(r_.e0, m->stream));                           \
+                L2_TRY(call);                                                       \
+                L2_HIP(hipEventRecord(r_.e1, m->stream));                           \
+            }                                                                       \
+            m->prof.push_back(r_);                                                  \
+        } else {                                                                    \
+            L2_TRY(call);                                                           \
+        }                                                                           \
     } while (0)
 
 struct l2_state {

@@ -229,7 +229,12 @@ int launch_t(Q4Launch &L, hipStream_t stream) {
         }
     }
     dim3 grid(total, L.batch), block(NW * 64);
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, L);
+    if (g_q4_prof.armed) {
+        g_q4_prof.armed = false;
+        hipExtLaunchKernelGGL(kern, grid, block, lds, stream, g_q4_prof.start, g_q4_prof.stop, 0, L);
+    } else {
+        hipLaunchKernelGGL(kern, grid, block, lds, stream, L);
+    }
     L2_HIP(hipGetLastError());
     return L2_OK;
 }

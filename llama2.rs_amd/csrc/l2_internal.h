@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -81,6 +82,15 @@ struct Q4Launch {
     float eps;   // rmsnorm epsilon, used when wn is set
     int rows_per_block; // filled by the streaming launcher
 };
+
+// When armed (profiling runs only), the next q4 launch goes out through
+// hipExtLaunchKernel with these events, which then carry the dispatch's own
+// begin and end timestamps rather than those of marker packets around it.
+struct Q4ProfHook {
+    hipEvent_t start = nullptr, stop = nullptr;
+    bool armed = false;
+};
+extern thread_local Q4ProfHook g_q4_prof;
 
 // Launch the fp32 dequant matvec for up to 3 matrices that share `in`
 // (wq|wk|wv), or a (w1, w3) pair.  Fills row_blocks itself.
