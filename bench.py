@@ -63,6 +63,57 @@ def token_bytes(d, pos: int) -> int:
     return d.n_layers * per_layer + cb["classifier"] + d.dim * 4 + d.dim * 4 + kv
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix peak
+
+
+def prefill_workload(a, d, m, img, np) -> int:
+    """BASELINE config 2: a prompt of --prompt-len random ids prefilled in chunks of --chunk tokens
+    through the dequant->fp16 MFMA GEMM path, followed by --steps greedy decode steps."""
+    from llama2_rs import _lib
+    n, chunk, K = a.prompt_len, a.chunk, a.steps
+    rng = np.random.default_rng(a.seed)
+    prompt = rng.integers(0, d.vocab_size, size=n).astype(np.int32)
+    flops_per_token = 2 * d.n_layers * (2 * d.dim * d.dim + 2 * d.dim * d.kv_dim + 3 * d.dim * d.hidden_dim)
+
+    def run(mode):
+        m.set_prefill_mode(mode)
+        m.reset()
+        m.forward(prompt[:min(chunk, n)], np.arange(min(chunk, n), dtype=np.int32))  # warm-up chunk
+        m.reset()
+        t0 = time.perf_counter()
+        for c0 in range(0, n, chunk):
+            c1 = min(c0 + chunk, n)
+            toks = np.concatenate([[1], prompt[:c1 - 1]])[c0:c1].astype(np.int32)  # START-shifted, as prefill<A> does
+            m.forward(toks, np.arange(c0, c1, dtype=np.int32))
+        return time.perf_counter() - t0
+
+    t_mfma = run(_lib.PREFILL_MFMA)
+    ids, ms_dec = m.decode_bench(int(prompt[-1]), n, K)
+    t_fp32 = run(_lib.PREFILL_FP32) if a.cpu_tokens >= 0 else None
+    ids32, _ = m.decode_bench(int(prompt[-1]), n, K)
+    same = int(np.sum(np.cumprod(ids == ids32)))
+    tok_s = n / t_mfma
+    tflops = flops_per_token * tok_s / 1e12
+    result = {
+        "metric": f"{a.model} q4 prefill tok/s on 1 MI355X", "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1,
+        "steps": n // chunk, "warmup": 1, "ms_per_step": round(t_mfma * 1e3 / max(1, (n + chunk - 1) // chunk), 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 x f16 -> f32 (MFMA)",
+        "data": "synthetic",
+        "config": {"workload": f"Llama-2-{a.model} GPTQ 4-bit group {d.group_size} act-order, random-init; {n}-token random "
+                               f"prompt prefilled in chunks of {chunk} through the dequant->fp16 MFMA GEMM, then {K} greedy steps",
+                   "seed": a.seed},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "flops_per_token": flops_per_token},
+        "fp32_path_tok_s": round(n / t_fp32, 1) if t_fp32 else None,
+        "decode_after_prefill_tok_s": round(K / (ms_dec * 1e-3), 1),
+        "greedy_tokens_same_as_after_fp32_prefill": f"{same}/{K}",
+    }
+    m.close()
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,6 +126,10 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="decoded tokens of the CPU sample (0 = sized to ~20 s)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
+                    help="prefill: BASELINE config 2 (prompt in chunks through the dequant->fp16 MFMA GEMM, then decode)")
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--chunk", type=int, default=128)
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no sharding, no collectives); "
@@ -97,6 +152,9 @@ def main() -> int:
     t0 = time.time()
     m = ops.Model(img, d, max_seq=max_seq)
     t_upload = time.time() - t0
+
+    if a.workload == "prefill":
+        return prefill_workload(a, d, m, img, np)
 
     rng = np.random.default_rng(a.seed)
     prompt = rng.integers(0, d.vocab_size, size=W).astype(np.int32)

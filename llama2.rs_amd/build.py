@@ -25,6 +25,7 @@ SOURCES = {
     # file: extra flags
     "kernels_q4.hip": [],
     "kernels_q4_stream.hip": [],
+    "kernels_q4_gemm.hip": [],
     # the block kernels keep the reference's rounded-multiply-then-add where they restate it
     "kernels_misc.hip": ["-ffp-contract=off"],
     "host.cpp": ["-x", "hip", "-ffp-contract=off"],

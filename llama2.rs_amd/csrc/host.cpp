@@ -281,6 +281,10 @@ struct l2_model {
     int cap_B = 0;
     float *x = nullptr, *xq = nullptr, *xk = nullptr, *xv = nullptr, *qv = nullptr, *kv = nullptr,
           *vv = nullptr, *attg = nullptr, *x1 = nullptr, *x3 = nullptr, *hg = nullptr, *logits = nullptr;
+    // extra scratch of the MFMA prefill path (cap_B_mfma columns): fp16 inputs, w1/w3 outputs, row scales
+    int cap_B_mfma = 0;
+    void *h16a = nullptr, *h16b = nullptr, *h16c = nullptr; // fp16 [B][max(dim, hidden)]
+    float *hb = nullptr, *hb2 = nullptr, *ssb = nullptr;
     int32_t *dtok = nullptr, *dpos = nullptr;
     unsigned long long *amax = nullptr;
     int32_t *dprompt = nullptr, *dout_ids = nullptr;
@@ -592,7 +596,8 @@ extern "C" void l2_model_close(l2_model *m) {
     if (m->stream) (void)hipStreamSynchronize(m->stream);
     void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->dwn, m->attn_part, m->x, m->xq, m->xk,
                     m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->logits, m->dtok, m->dpos,
-                    m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y};
+                    m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y, m->h16a, m->h16b, m->h16c,
+                    m->hb, m->hb2, m->ssb};
     for (void *p : ptrs) dfree(p);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
@@ -616,10 +621,15 @@ extern "C" int l2_prefill_supported(const l2_model *m) { return m ? 1 : 0; }
 
 extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
     if (!m) return l2_fail(L2_ERR_ARG, "null model");
-    if (mode != L2_PREFILL_FP32) return l2_fail(L2_ERR_ARG, "prefill mode %d is not available", mode);
+    if (mode != L2_PREFILL_FP32 && mode != L2_PREFILL_MFMA) return l2_fail(L2_ERR_ARG, "prefill mode %d", mode);
+    if (mode == L2_PREFILL_MFMA && !(q4_gemm_supports(m->d.dim, m->d.dim) && q4_gemm_supports(m->d.hidden_dim, m->kv_dim) &&
+                                     q4_gemm_supports(m->d.dim, m->d.hidden_dim)))
+        return l2_fail(L2_ERR_ARG, "the MFMA prefill path needs dim and hidden_dim to be multiples of 64");
     m->prefill_mode = mode;
     return L2_OK;
 }
+
+static int ensure_batch_mfma(l2_model *m, int B);
 
 static int ensure_batch(l2_model *m, int B) {
     if (B <= m->cap_B) return L2_OK;
@@ -863,6 +873,21 @@ extern "C" int l2_model_qmatvec(l2_model *m, int layer, int proj, const float *x
     if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
     const DevQLinear &q = m->q[proj][layer];
     L2_TRY(op_scratch(m, (size_t)B * std::max(std::max(q.in, q.out), m->d.vocab_size)));
+    if (B > 1 && m->prefill_mode == L2_PREFILL_MFMA && q4_gemm_supports(q.in, q.out)) {
+        // the prefill form of the same operator: gather, round to fp16, dequant -> MFMA
+        hipStream_t st = m->stream;
+        L2_TRY(ensure_batch_mfma(m, B));
+        L2_HIP(hipMemcpyAsync(m->op_x, x_host, (size_t)B * q.in * 4, hipMemcpyHostToDevice, st));
+        L2_TRY(gather_launch(m->op_xg, m->op_x, q.g_index, q.in, B, st));
+        L2_TRY(prep_f16_launch(m->h16a, m->op_xg, nullptr, q.in, B, st));
+        Q4Launch Q = launch_of(q, B, 0.f);
+        Q.m[0] = mat_of(q, nullptr, nullptr, m->op_y);
+        XhList X{{m->h16a, nullptr, nullptr}};
+        L2_TRY(q4_gemm_launch(Q, X, nullptr, st));
+        L2_HIP(hipMemcpyAsync(y_host, m->op_y, (size_t)B * q.out * 4, hipMemcpyDeviceToHost, st));
+        L2_HIP(hipStreamSynchronize(st));
+        return L2_OK;
+    }
     return matvec_host(q, m->op_x, m->op_xg, m->op_y, x_host, B, y_host, m->stream);
 }
 
@@ -990,6 +1015,113 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
     return L2_OK;
 }
 
+static int ensure_batch_mfma(l2_model *m, int B) {
+    if (B <= m->cap_B_mfma) return L2_OK;
+    L2_HIP(hipStreamSynchronize(m->stream));
+    void **bufs[] = {&m->h16a, &m->h16b, &m->h16c, (void **)&m->hb, (void **)&m->hb2, (void **)&m->ssb};
+    for (void **b : bufs) {
+        dfree(*b);
+        *b = nullptr;
+    }
+    m->cap_B_mfma = 0;
+    const size_t wide = (size_t)std::max(m->d.dim, m->d.hidden_dim);
+    uint16_t *p = nullptr;
+    L2_TRY(dalloc(&p, B * wide));
+    m->h16a = p;
+    L2_TRY(dalloc(&p, B * wide));
+    m->h16b = p;
+    L2_TRY(dalloc(&p, B * wide));
+    m->h16c = p;
+    L2_TRY(dalloc(&m->hb, B * (size_t)m->d.hidden_dim));
+    L2_TRY(dalloc(&m->hb2, B * (size_t)m->d.hidden_dim));
+    L2_TRY(dalloc(&m->ssb, (size_t)B));
+    m->cap_B_mfma = B;
+    return L2_OK;
+}
+
+// A prefill chunk through the matrix cores: the same schedule as forward_enqueue,
+// with every QLinear as a dequant -> fp16 -> MFMA GEMM over the B tokens and the
+// element-wise steps as kernels of their own.  Logits are never produced here
+// (src/models.rs:288).
+static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
+    const l2_dims &d = m->d;
+    const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
+    hipStream_t st = m->stream;
+    L2_TRY(ensure_batch_mfma(m, B));
+    {
+        ScatterTargets t{};
+        t.n = 3;
+        t.inv[0] = m->q[L2_WQ][0].inv_index, t.inv[1] = m->q[L2_WK][0].inv_index, t.inv[2] = m->q[L2_WV][0].inv_index;
+        t.out[0] = m->xq, t.out[1] = m->xk, t.out[2] = m->xv;
+        L2_TRY(embed_launch(m->x, m->tok_emb, m->dtok, dim, B, t, m->amax, st));
+    }
+    for (int l = 0; l < L; l++) {
+        const DevQLinear &wq = m->q[L2_WQ][l], &wk = m->q[L2_WK][l], &wv = m->q[L2_WV][l],
+                         &wo = m->q[L2_WO][l], &w1 = m->q[L2_W1][l], &w2 = m->q[L2_W2][l],
+                         &w3 = m->q[L2_W3][l];
+        const float *wn = m->dwn + (size_t)l * 5 * dim;
+        L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
+        L2_TRY(prep_f16_launch(m->h16a, m->xq, wn + 0 * (size_t)dim, dim, B, st));
+        L2_TRY(prep_f16_launch(m->h16b, m->xk, wn + 1 * (size_t)dim, dim, B, st));
+        L2_TRY(prep_f16_launch(m->h16c, m->xv, wn + 2 * (size_t)dim, dim, B, st));
+        {
+            Q4Launch Q = launch_of(wq, B, m->rms_eps);
+            Q.m[0] = mat_of(wq, nullptr, nullptr, m->qv);
+            Q.m[1] = mat_of(wk, nullptr, nullptr, m->kv);
+            Q.m[2] = mat_of(wv, nullptr, nullptr, m->vv);
+            Q.n_mats = 3;
+            XhList X{{m->h16a, m->h16b, m->h16c}};
+            L2_TRY(q4_gemm_launch(Q, X, m->ssb, st));
+        }
+        float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
+        float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
+        L2_TRY(rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
+                              d.n_kv_heads, m->head_size, B, st));
+        L2_TRY(attention_launch(m->attg, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
+                                m->head_size, max_pos, B, st));
+        L2_TRY(prep_f16_launch(m->h16a, m->attg, nullptr, dim, B, st));
+        {
+            Q4Launch Q = launch_of(wo, B, 0.f);
+            Q.m[0] = mat_of(wo, nullptr, nullptr, m->x);
+            Q.e.kind = Q4_EPI_RESIDUAL;
+            Q.e.res = m->x;
+            Q.e.n_scatter = 2;
+            Q.e.sc_idx[0] = w1.inv_index, Q.e.sc_out[0] = m->x1;
+            Q.e.sc_idx[1] = w3.inv_index, Q.e.sc_out[1] = m->x3;
+            XhList X{{m->h16a, nullptr, nullptr}};
+            L2_TRY(q4_gemm_launch(Q, X, nullptr, st));
+        }
+        L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
+        L2_TRY(prep_f16_launch(m->h16a, m->x1, wn + 3 * (size_t)dim, dim, B, st));
+        L2_TRY(prep_f16_launch(m->h16b, m->x3, wn + 4 * (size_t)dim, dim, B, st));
+        {
+            Q4Launch Q = launch_of(w1, B, m->rms_eps);
+            Q.m[0] = mat_of(w1, nullptr, nullptr, m->hb);
+            Q.m[1] = mat_of(w3, nullptr, nullptr, m->hb2);
+            Q.n_mats = 2;
+            XhList X{{m->h16a, m->h16b, nullptr}};
+            L2_TRY(q4_gemm_launch(Q, X, m->ssb, st));
+        }
+        L2_TRY(silu_scatter_launch(m->hg, m->hb, m->hb2, w2.inv_index, hid, B, st));
+        L2_TRY(prep_f16_launch(m->h16a, m->hg, nullptr, hid, B, st));
+        {
+            Q4Launch Q = launch_of(w2, B, 0.f);
+            Q.m[0] = mat_of(w2, nullptr, nullptr, m->x);
+            Q.e.kind = Q4_EPI_RESIDUAL;
+            Q.e.res = m->x;
+            if (l + 1 < L) {
+                Q.e.n_scatter = 3;
+                Q.e.sc_idx[0] = m->q[L2_WQ][l + 1].inv_index, Q.e.sc_out[0] = m->xq;
+                Q.e.sc_idx[1] = m->q[L2_WK][l + 1].inv_index, Q.e.sc_out[1] = m->xk;
+                Q.e.sc_idx[2] = m->q[L2_WV][l + 1].inv_index, Q.e.sc_out[2] = m->xv;
+            }
+            XhList X{{m->h16a, nullptr, nullptr}};
+            L2_TRY(q4_gemm_launch(Q, X, nullptr, st));
+        }
+    }
+    return L2_OK;
+}
+
 static int check_tokens(const l2_model *m, const int32_t *tokens, const int32_t *pos, int B, int *max_pos) {
     int mp = 0;
     for (int b = 0; b < B; b++) {
@@ -1013,7 +1145,10 @@ extern "C" int l2_forward(l2_model *m, l2_state *s, const int32_t *tokens, const
     L2_TRY(ensure_batch(m, B));
     L2_HIP(hipMemcpyAsync(m->dtok, tokens, (size_t)B * 4, hipMemcpyHostToDevice, m->stream));
     L2_HIP(hipMemcpyAsync(m->dpos, pos, (size_t)B * 4, hipMemcpyHostToDevice, m->stream));
-    L2_TRY(forward_enqueue(m, s, B, max_pos, B == 1));
+    if (B > 1 && m->prefill_mode == L2_PREFILL_MFMA)
+        L2_TRY(forward_enqueue_mfma(m, s, B, max_pos));
+    else
+        L2_TRY(forward_enqueue(m, s, B, max_pos, B == 1));
     if (B == 1 && logits_host)
         L2_HIP(hipMemcpyAsync(logits_host, m->logits, (size_t)m->d.vocab_size * 4, hipMemcpyDeviceToHost, m->stream));
     L2_HIP(hipStreamSynchronize(m->stream));
@@ -1096,7 +1231,10 @@ extern "C" int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *promp
                 }
                 L2_HIP(hipMemcpyAsync(m->dtok, toks.data(), (size_t)A * 4, hipMemcpyHostToDevice, m->stream));
                 L2_HIP(hipMemcpyAsync(m->dpos, poss.data(), (size_t)A * 4, hipMemcpyHostToDevice, m->stream));
-                L2_TRY(forward_enqueue(m, s, A, pos - 1, false));
+                if (m->prefill_mode == L2_PREFILL_MFMA)
+                    L2_TRY(forward_enqueue_mfma(m, s, A, pos - 1));
+                else
+                    L2_TRY(forward_enqueue(m, s, A, pos - 1, false));
                 L2_HIP(hipStreamSynchronize(m->stream)); // toks/poss are reused
             }
         }

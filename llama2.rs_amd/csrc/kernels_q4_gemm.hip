@@ -1,0 +1,361 @@
+// Batched-prefill form of the GPTQ 4-bit linear layer for gfx950: dequantise
+// tiles of the packed weights to fp16 in registers and feed them to the matrix
+// cores (v_mfma_f32_32x32x16_f16), fp32 accumulate.
+//
+//   Y[t][o] = sum_k W[o][k] * X[t][k],   W[o][k] = scales[o][k/G] * (nib(qweight[o],k) - z1[o][k/G])
+//
+// for a chunk of T tokens whose inputs the caller has already brought into this
+// layer's g_index order, multiplied by the norm weight where one applies, and
+// rounded to fp16 (prep_f16_kernel).  This is the one place in the token loop
+// that is a dense contraction, hence the one place that uses MFMA; the decode
+// matvec stays on the vector ALU in fp32.
+//
+// Tiling.  A block is 4 waves; a wave owns MT=2 tiles of 32 output rows and all
+// NB blocks of 32 tokens, so a block covers 256 rows x 32*NB tokens.  K advances
+// 64 at a time: lane (r = l%32, h = l/32) loads the 16 bytes qweight[o][K/8+4h ..
+// +4) of its row -- four packed words, each of which is exactly the 8 k-values
+// one MFMA step wants from this lane.  The X slice [tokens][64] is staged in LDS
+// (rows padded to 72 halves so that 16-byte reads of 32 lanes are conflict-free),
+// double-buffered.
+//
+// Dequant.  (w >> 4i) & 0x000F000F | 0x64006400 is the fp16 pair (1024+n_i,
+// 1024+n_{i+4}); subtracting 1024+z1 is exact.  The pairs come out as
+// (n0,n4),(n1,n5),(n2,n6),(n3,n7), so X is stored with the same interleave
+// inside every 8 consecutive k.  For G >= 64 the matrix cores see the exact
+// integers n - z1 and the fp32 scale is applied to the fp32 partial sum of each
+// group (one FMA per accumulator element and group), so the only rounding on
+// the weight side is none at all; for G = 32 a K step of 64 straddles two
+// groups, and the weights are multiplied by fp16(scale) before the MFMA.
+#include "l2_internal.h"
+
+namespace {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int kXRow = 72; // halves per staged token row: 64 + 8 pad
+
+union A8 {
+    h8 v;
+    h2 p[4];
+    uint32_t u[4];
+};
+
+// One packed word of 8 nibbles -> 8 fp16 values n - z1 (exact), times `scale` if
+// SCALED, in the pair order (0,4,1,5,2,6,3,7).
+template <bool SCALED>
+__device__ __forceinline__ h8 dequant8(uint32_t w, h2 neg_off, h2 scale) {
+    A8 a;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t t = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+        h2 v = __builtin_bit_cast(h2, t);
+        v = v + neg_off; // (1024 + n) - (1024 + z1), exact
+        a.p[i] = SCALED ? v * scale : v;
+    }
+    return a.v;
+}
+
+template <int G, int NB>
+__global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss) {
+    constexpr int MT = 2;
+    constexpr int TN = 32 * NB;
+    constexpr bool SA = G >= 64; // scale after the group's partial sum
+    extern __shared__ _Float16 xs[]; // [2][TN][kXRow]
+    __shared__ float gsc[2][256];    // fp32 scales of the block's 256 rows for the current group
+    const int in = L.in;
+    const int n_k = in >> 6; // K iterations of 64
+
+    int rb = blockIdx.x;
+    int mi = 0;
+    while (mi + 1 < L.n_mats && rb >= L.m[mi].row_blocks) {
+        rb -= L.m[mi].row_blocks;
+        mi++;
+    }
+    const Q4Mat &M = L.m[mi];
+    const _Float16 *xh = reinterpret_cast<const _Float16 *>(xh_list.p[mi]); // [B][in] fp16, pair-interleaved
+    const int n_out = M.out;
+    const int groups = L.groups;
+    const int B = L.batch;
+    const int t0 = blockIdx.y * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int C4 = in >> 5; // uint4 per weight row
+
+    int orow[MT];
+    bool live[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int o = (rb * 4 + wave) * (32 * MT) + mt * 32 + r;
+        live[mt] = o < n_out;
+        orow[mt] = live[mt] ? o : n_out - 1;
+    }
+
+    f16v acc[MT][NB];  // running result
+    f16v accg[MT][NB]; // partial sum of the current group (SA only)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                acc[mt][nb][i] = 0.f;
+                accg[mt][nb][i] = 0.f;
+            }
+    constexpr int KPG = G / 64 > 0 ? G / 64 : 1; // K iterations per group
+    auto load_group_scales = [&](int g, int buf) {
+        const int o = rb * 256 + tid;
+        gsc[buf][tid] = o < n_out ? M.scales[(size_t)o * groups + g] : 0.f;
+    };
+
+    // staging map: thread -> (token, 16-byte segment) x (TN*8/256) pieces
+    constexpr int PIECES = TN * 8 / 256;
+    uint4 stage[PIECES];
+    auto load_stage = [&](int kit) {
+#pragma unroll
+        for (int p = 0; p < PIECES; p++) {
+            const int idx = p * 256 + tid;
+            const int t = idx >> 3, seg = idx & 7;
+            const int tg = t0 + t;
+            stage[p] = tg < B ? *reinterpret_cast<const uint4 *>(xh + (size_t)tg * in + (size_t)kit * 64 + seg * 8)
+                              : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto store_stage = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < PIECES; p++) {
+            const int idx = p * 256 + tid;
+            const int t = idx >> 3, seg = idx & 7;
+            *reinterpret_cast<uint4 *>(xs + ((size_t)buf * TN + t) * kXRow + seg * 8) = stage[p];
+        }
+    };
+
+    uint4 wq[MT];
+    float sc[MT];
+    int32_t zw[MT];
+    auto load_w = [&](int kit) {
+        const int g = (kit * 64 + 32 * h) / G;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            wq[mt] = M.qweight[(size_t)orow[mt] * C4 + kit * 2 + h];
+            sc[mt] = M.scales[(size_t)orow[mt] * groups + g];
+            zw[mt] = M.qzeros[(size_t)(orow[mt] >> 3) * groups + g];
+        }
+    };
+
+    load_stage(0);
+    load_w(0);
+    store_stage(0);
+    if (SA) load_group_scales(0, 0);
+    __syncthreads();
+
+    for (int kit = 0; kit < n_k; kit++) {
+        const int buf = kit & 1;
+        // this iteration's weights -> registers of their own, then request the next
+        uint4 wc[MT];
+        h2 noff[MT], s16[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            wc[mt] = wq[mt];
+            const int zn = (zw[mt] >> (4 * (orow[mt] & 7))) & 15;
+            const _Float16 off = (_Float16)(-(1024.0f + (float)(zn + 1)));
+            noff[mt] = h2{off, off};
+            const _Float16 s = (_Float16)sc[mt];
+            s16[mt] = h2{s, s};
+        }
+        if (kit + 1 < n_k) {
+            load_stage(kit + 1);
+            load_w(kit + 1);
+        }
+        const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h8 a[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                const uint32_t word = j == 0 ? wc[mt].x : j == 1 ? wc[mt].y : j == 2 ? wc[mt].z : wc[mt].w;
+                a[mt] = dequant8<!SA>(word, noff[mt], s16[mt]);
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                const h8 b = *reinterpret_cast<const h8 *>(xb + (size_t)(nb * 32 + r) * kXRow + (4 * h + j) * 8);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    if (SA)
+                        accg[mt][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, accg[mt][nb], 0, 0, 0);
+                    else
+                        acc[mt][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, acc[mt][nb], 0, 0, 0);
+                }
+            }
+        }
+        if (SA && (kit + 1) % KPG == 0) {
+            // end of a group: fold its partial sum into the result with the fp32 scale of each row
+            const int gb = (kit / KPG) & 1;
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][wave * 64 + mt * 32 + q * 8 + h * 4]);
+                    const float svv[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            acc[mt][nb][4 * q + e] = fmaf(svv[e], accg[mt][nb][4 * q + e], acc[mt][nb][4 * q + e]);
+                            accg[mt][nb][4 * q + e] = 0.f;
+                        }
+                }
+            if (kit + 1 < n_k) load_group_scales((kit + 1) / KPG, gb ^ 1);
+        }
+        if (kit + 1 < n_k) store_stage(buf ^ 1);
+        __syncthreads();
+    }
+
+    // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4
+    const Q4Epi &E = L.e;
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int obase = (rb * 4 + wave) * (32 * MT) + mt * 32;
+        if (obase >= n_out) continue;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const int t = t0 + nb * 32 + r;
+            if (t >= B) continue;
+            const float scale_t = ss ? ss[t] : 1.0f;
+            const size_t row = (size_t)t * n_out;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int o = obase + q * 8 + h * 4;
+                float4 v = make_float4(acc[mt][nb][4 * q + 0] * scale_t, acc[mt][nb][4 * q + 1] * scale_t,
+                                       acc[mt][nb][4 * q + 2] * scale_t, acc[mt][nb][4 * q + 3] * scale_t);
+                if (E.kind == Q4_EPI_RESIDUAL) {
+                    const float4 rr = *reinterpret_cast<const float4 *>(E.res + row + o);
+                    v.x += rr.x;
+                    v.y += rr.y;
+                    v.z += rr.z;
+                    v.w += rr.w;
+                }
+                if (E.kind != Q4_EPI_SCATTER_ONLY) *reinterpret_cast<float4 *>(M.y + row + o) = v;
+                const float vals[4] = {v.x, v.y, v.z, v.w};
+                for (int c = 0; c < E.n_scatter; c++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) E.sc_out[c][row + E.sc_idx[c][o + e]] = vals[e];
+            }
+        }
+    }
+}
+
+// fp32 [B][n] (already in the consumer's g_index order) -> fp16 [B][n], times the
+// norm weight if given, with the (0,4,1,5,2,6,3,7) interleave inside every 8.
+__global__ void prep_f16_kernel(_Float16 *out, const float *x, const float *wn, int n) {
+    const int b = blockIdx.y;
+    const int j8 = blockIdx.x * blockDim.x + threadIdx.x; // group of 8
+    if (j8 * 8 >= n) return;
+    const float4 a = reinterpret_cast<const float4 *>(x + (size_t)b * n)[j8 * 2];
+    const float4 c = reinterpret_cast<const float4 *>(x + (size_t)b * n)[j8 * 2 + 1];
+    float v[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
+    if (wn) {
+        const float4 g0 = reinterpret_cast<const float4 *>(wn)[j8 * 2];
+        const float4 g1 = reinterpret_cast<const float4 *>(wn)[j8 * 2 + 1];
+        const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] *= g[i];
+    }
+    A8 o;
+    o.p[0] = h2{(_Float16)v[0], (_Float16)v[4]};
+    o.p[1] = h2{(_Float16)v[1], (_Float16)v[5]};
+    o.p[2] = h2{(_Float16)v[2], (_Float16)v[6]};
+    o.p[3] = h2{(_Float16)v[3], (_Float16)v[7]};
+    reinterpret_cast<uint4 *>(out + (size_t)b * n)[j8] = make_uint4(o.u[0], o.u[1], o.u[2], o.u[3]);
+}
+
+// ss[b] = 1 / sqrt(mean(x[b]^2) + eps)   (src/models.rs:55-60)
+__global__ __launch_bounds__(256) void rms_scale_kernel(float *ss, const float *x, float eps, int dim) {
+    __shared__ float red[4];
+    const int b = blockIdx.x;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float v = x[(size_t)b * dim + i];
+        s = fmaf(v, v, s);
+    }
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = red[0] + red[1] + red[2] + red[3];
+        t /= (float)dim;
+        t += eps;
+        ss[b] = 1.0f / sqrtf(t);
+    }
+}
+
+// silu gate (src/models.rs:92-98) for a chunk: out[b][scatter[i]] = silu(a[b][i]) * c[b][i]
+__global__ void silu_scatter_kernel(float *out, const float *a, const float *c, const int32_t *scatter, int n) {
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = a[(size_t)b * n + i];
+    s = s * (1.0f / (1.0f + expf(-s)));
+    s = s * c[(size_t)b * n + i];
+    out[(size_t)b * n + (scatter ? scatter[i] : i)] = s;
+}
+
+template <int G>
+int launch_gemm_g(Q4Launch &L, const XhList &xh_list_dev, const float *ss, hipStream_t st) {
+    int total = 0;
+    for (int i = 0; i < L.n_mats; i++) {
+        L.m[i].row_blocks = (L.m[i].out + 255) / 256;
+        total += L.m[i].row_blocks;
+    }
+    const int B = L.batch;
+    const int NB = B > 64 ? 4 : B > 32 ? 2 : 1;
+    const int TN = 32 * NB;
+    dim3 grid(total, (B + TN - 1) / TN), block(256);
+    const size_t lds = (size_t)2 * TN * kXRow * sizeof(_Float16);
+    switch (NB) {
+        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1>), grid, block, lds, st, L, xh_list_dev, ss); break;
+        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2>), grid, block, lds, st, L, xh_list_dev, ss); break;
+        default: hipLaunchKernelGGL((q4_gemm_kernel<G, 4>), grid, block, lds, st, L, xh_list_dev, ss); break;
+    }
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+} // namespace
+
+int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, hipStream_t st) {
+    if (L.n_mats < 1 || L.n_mats > 3) return l2_fail(L2_ERR_ARG, "q4 gemm: n_mats=%d", L.n_mats);
+    if (L.in % 64 != 0 || L.in % L.group_size != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d must be a multiple of 64", L.in);
+    for (int i = 0; i < L.n_mats; i++)
+        if (L.m[i].out % 32 != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: out=%d must be a multiple of 32", L.m[i].out);
+    if (L.pair) return l2_fail(L2_ERR_ARG, "q4 gemm: pair launches are not supported");
+    switch (L.group_size) {
+        case 32: return launch_gemm_g<32>(L, xh_list_dev, ss, st);
+        case 64: return launch_gemm_g<64>(L, xh_list_dev, ss, st);
+        case 128: return launch_gemm_g<128>(L, xh_list_dev, ss, st);
+    }
+    return l2_fail(L2_ERR_ARG, "q4 gemm: group size %d", L.group_size);
+}
+
+bool q4_gemm_supports(int in, int out) { return in % 64 == 0 && out % 32 == 0; }
+
+int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st) {
+    if (n % 8) return l2_fail(L2_ERR_ARG, "prep: n=%d not a multiple of 8", n);
+    hipLaunchKernelGGL(prep_f16_kernel, dim3((n / 8 + 255) / 256, B), dim3(256), 0, st, (_Float16 *)out_f16, x, wn, n);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int rms_scale_launch(float *ss, const float *x, float eps, int dim, int B, hipStream_t st) {
+    hipLaunchKernelGGL(rms_scale_kernel, dim3(B), dim3(256), 0, st, ss, x, eps, dim);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int silu_scatter_launch(float *out, const float *a, const float *c, const int32_t *scatter, int n, int B,
+                        hipStream_t st) {
+    hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, a, c, scatter, n);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}

@@ -99,6 +99,21 @@ int q4_matvec_launch(Q4Launch &L, hipStream_t stream);
 int q4_stream_launch(Q4Launch &L, hipStream_t stream);
 bool q4_stream_supports(const Q4Launch &L);
 
+// ---- prefill chunks through the matrix cores ---------------------------------
+
+struct XhList {
+    const void *p[3]; // per matrix of the launch: fp16 [B][in], g_index order, pair-interleaved (prep_f16_launch)
+};
+// Y = X W^T for a chunk of L.batch tokens; ss (per token, may be null) scales the rows of Y.
+// Epilogues as in the matvec (no pair launches).
+int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, hipStream_t st);
+bool q4_gemm_supports(int in, int out);
+// out_f16[b][j'] = fp16(x[b][j] * (wn ? wn[j] : 1)), j' = j with the order (0,4,1,5,2,6,3,7) inside every 8.
+int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st);
+int rms_scale_launch(float *ss, const float *x, float eps, int dim, int B, hipStream_t st);
+int silu_scatter_launch(float *out, const float *a, const float *c, const int32_t *scatter, int n, int B,
+                        hipStream_t st);
+
 // ---- the other per-token kernels -------------------------------------------
 
 struct ScatterTargets {

@@ -142,6 +142,10 @@ class Model:
     def reset(self):
         check(lib().l2_state_reset(self.state))
 
+    def set_prefill_mode(self, mode: int):
+        """_lib.PREFILL_FP32 (default, identical to B=1) or _lib.PREFILL_MFMA (fp16 tiles, 2e-3)."""
+        check(lib().l2_model_set_prefill_mode(self.h, mode))
+
     def qmatvec(self, layer: int, proj: int, x) -> np.ndarray:
         x = _f32(x)
         one = x.ndim == 1

@@ -250,3 +250,46 @@ def test_text_generate_api(ops, oracle, tmp_path):
     assert a == b and len(a) == len(c)
     model.close()
     o.close()
+
+
+REL_MFMA = 2e-3   # fp16 tiles into MFMA, fp32 accumulate
+
+
+@pytest.mark.parametrize("dims,B", [(TINY_GQA, 5), (MID, 33), (MID, 128)], ids=["gqa_g128_b5", "g32_b33", "g32_b128"])
+def test_mfma_prefill_operator_and_forward(ops, oracle, dims, B):
+    """The dequant->fp16->MFMA form of QLinear::matvec<B> and of transformer<B> (B > 1)."""
+    from llama2_rs import _lib
+    img = ck.synth_weights_image(dims, seed=5)
+    m = ops.Model(img, dims)
+    o = oracle.Model(img, dims)
+    m.set_prefill_mode(_lib.PREFILL_MFMA)
+    rng = np.random.default_rng(B)
+    import tests.test_oracle_loop as tol
+    W = tol._split_image(img, dims)
+    x = rng.standard_normal((B, dims.dim)).astype(np.float32)
+    hx = rng.standard_normal((B, dims.hidden_dim)).astype(np.float32)
+    for proj, name, xin in ((_lib.WQ, "wq", x), (_lib.WK, "wk", x), (_lib.W1, "w1", x), (_lib.W2, "w2", hx)):
+        got = m.qmatvec(0, proj, xin)
+        want = (W[name][0] @ xin.astype(np.float64).T).T
+        assert nrel(got, want) < REL_MFMA, name
+        fp32 = ops.Model(img, dims)
+        assert nrel(got, fp32.qmatvec(0, proj, xin)) < REL_MFMA
+        fp32.close()
+    # a chunk of B positions through the whole layer stack: cache rows and the logits that follow
+    n = min(B, dims.seq_len - 2)
+    toks = rng.integers(0, dims.vocab_size, size=n).astype(np.int32)
+    poss = np.arange(n, dtype=np.int32)
+    m.reset()
+    m.forward(toks, poss)
+    o.new_state()
+    o.transformer(toks, poss)
+    ko, vo = o.kv_cache()
+    for l in range(dims.n_layers):
+        k, v = m.read_kv(l, 0, n)
+        assert nrel(k, ko[l, :n]) < 5 * REL_MFMA
+        assert nrel(v, vo[l, :n]) < 5 * REL_MFMA
+    got = m.forward([7], [n])
+    want = o.transformer([7], [n])
+    assert nrel(got, want) < 5 * REL_MFMA
+    m.close()
+    o.close()
