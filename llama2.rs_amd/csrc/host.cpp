@@ -284,7 +284,8 @@ struct l2_model {
     // extra scratch of the MFMA prefill path (cap_B_mfma columns): fp16 inputs, w1/w3 outputs, row scales
     int cap_B_mfma = 0;
     void *h16a = nullptr, *h16b = nullptr, *h16c = nullptr; // fp16 [B][max(dim, hidden)]
-    float *hb = nullptr, *hb2 = nullptr, *ssb = nullptr;
+    float *hb = nullptr, *hb2 = nullptr, *ssb = nullptr, *gemm_ws = nullptr;
+    size_t gemm_ws_floats = 0;
     int32_t *dtok = nullptr, *dpos = nullptr;
     unsigned long long *amax = nullptr;
     int32_t *dprompt = nullptr, *dout_ids = nullptr;
@@ -597,7 +598,7 @@ extern "C" void l2_model_close(l2_model *m) {
     void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->dwn, m->attn_part, m->x, m->xq, m->xk,
                     m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->logits, m->dtok, m->dpos,
                     m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y, m->h16a, m->h16b, m->h16c,
-                    m->hb, m->hb2, m->ssb};
+                    m->hb, m->hb2, m->ssb, m->gemm_ws};
     for (void *p : ptrs) dfree(p);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
@@ -883,7 +884,7 @@ extern "C" int l2_model_qmatvec(l2_model *m, int layer, int proj, const float *x
         Q4Launch Q = launch_of(q, B, 0.f);
         Q.m[0] = mat_of(q, nullptr, nullptr, m->op_y);
         XhList X{{m->h16a, nullptr, nullptr}};
-        L2_TRY(q4_gemm_launch(Q, X, nullptr, st));
+        L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
         L2_HIP(hipMemcpyAsync(y_host, m->op_y, (size_t)B * q.out * 4, hipMemcpyDeviceToHost, st));
         L2_HIP(hipStreamSynchronize(st));
         return L2_OK;
@@ -1018,7 +1019,9 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
 static int ensure_batch_mfma(l2_model *m, int B) {
     if (B <= m->cap_B_mfma) return L2_OK;
     L2_HIP(hipStreamSynchronize(m->stream));
-    void **bufs[] = {&m->h16a, &m->h16b, &m->h16c, (void **)&m->hb, (void **)&m->hb2, (void **)&m->ssb};
+    void **bufs[] = {&m->h16a, &m->h16b, &m->h16c, (void **)&m->hb, (void **)&m->hb2, (void **)&m->ssb,
+                     (void **)&m->gemm_ws};
+    m->gemm_ws_floats = 0;
     for (void **b : bufs) {
         dfree(*b);
         *b = nullptr;
@@ -1035,6 +1038,9 @@ static int ensure_batch_mfma(l2_model *m, int B) {
     L2_TRY(dalloc(&m->hb, B * (size_t)m->d.hidden_dim));
     L2_TRY(dalloc(&m->hb2, B * (size_t)m->d.hidden_dim));
     L2_TRY(dalloc(&m->ssb, (size_t)B));
+    // split-K partial tiles: up to 8 slices of the widest launch (w1|w3 or q|k|v)
+    m->gemm_ws_floats = (size_t)8 * B * std::max((size_t)2 * m->d.hidden_dim, (size_t)m->d.dim + 2 * m->kv_dim) / 2;
+    L2_TRY(dalloc(&m->gemm_ws, m->gemm_ws_floats));
     m->cap_B_mfma = B;
     return L2_OK;
 }
@@ -1071,7 +1077,7 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
             Q.m[2] = mat_of(wv, nullptr, nullptr, m->vv);
             Q.n_mats = 3;
             XhList X{{m->h16a, m->h16b, m->h16c}};
-            L2_TRY(q4_gemm_launch(Q, X, m->ssb, st));
+            L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st));
         }
         float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
         float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
@@ -1089,7 +1095,7 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
             Q.e.sc_idx[0] = w1.inv_index, Q.e.sc_out[0] = m->x1;
             Q.e.sc_idx[1] = w3.inv_index, Q.e.sc_out[1] = m->x3;
             XhList X{{m->h16a, nullptr, nullptr}};
-            L2_TRY(q4_gemm_launch(Q, X, nullptr, st));
+            L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
         }
         L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
         L2_TRY(prep_f16_launch(m->h16a, m->x1, wn + 3 * (size_t)dim, dim, B, st));
@@ -1100,7 +1106,7 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
             Q.m[1] = mat_of(w3, nullptr, nullptr, m->hb2);
             Q.n_mats = 2;
             XhList X{{m->h16a, m->h16b, nullptr}};
-            L2_TRY(q4_gemm_launch(Q, X, m->ssb, st));
+            L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st));
         }
         L2_TRY(silu_scatter_launch(m->hg, m->hb, m->hb2, w2.inv_index, hid, B, st));
         L2_TRY(prep_f16_launch(m->h16a, m->hg, nullptr, hid, B, st));
@@ -1116,7 +1122,7 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
                 Q.e.sc_idx[2] = m->q[L2_WV][l + 1].inv_index, Q.e.sc_out[2] = m->xv;
             }
             XhList X{{m->h16a, nullptr, nullptr}};
-            L2_TRY(q4_gemm_launch(Q, X, nullptr, st));
+            L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
         }
     }
     return L2_OK;

@@ -10,8 +10,12 @@
 // that is a dense contraction, hence the one place that uses MFMA; the decode
 // matvec stays on the vector ALU in fp32.
 //
-// Tiling.  A block is 4 waves; a wave owns MT=2 tiles of 32 output rows and all
-// NB blocks of 32 tokens, so a block covers 256 rows x 32*NB tokens.  K advances
+// Tiling.  A block is 4 waves; a wave owns one tile of 32 output rows and all NB
+// blocks of 32 tokens (the dequantised weights are reused NB times), so a block
+// covers 128 rows x 32*NB tokens.  With only 128 tokens per chunk that leaves
+// few blocks, so K is also cut into KS slices across grid.z; each slice writes
+// its fp32 partial tile to a workspace and q4_gemm_reduce_kernel adds the
+// slices in a fixed order and runs the epilogue.  K advances
 // 64 at a time: lane (r = l%32, h = l/32) loads the 16 bytes qweight[o][K/8+4h ..
 // +4) of its row -- four packed words, each of which is exactly the 8 k-values
 // one MFMA step wants from this lane.  The X slice [tokens][64] is staged in LDS
@@ -58,12 +62,13 @@ __device__ __forceinline__ h8 dequant8(uint32_t w, h2 neg_off, h2 scale) {
 }
 
 template <int G, int NB>
-__global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss) {
-    constexpr int MT = 2;
+__global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
+                                                      float *__restrict__ ws, int KS) {
+    constexpr int MT = 1;
     constexpr int TN = 32 * NB;
     constexpr bool SA = G >= 64; // scale after the group's partial sum
     extern __shared__ _Float16 xs[]; // [2][TN][kXRow]
-    __shared__ float gsc[2][256];    // fp32 scales of the block's 256 rows for the current group
+    __shared__ float gsc[2][128];    // fp32 scales of the block's 128 rows for the current group
     const int in = L.in;
     const int n_k = in >> 6; // K iterations of 64
 
@@ -87,7 +92,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     bool live[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-        const int o = (rb * 4 + wave) * (32 * MT) + mt * 32 + r;
+        const int o = rb * 128 + wave * 32 + mt * 32 + r;
         live[mt] = o < n_out;
         orow[mt] = live[mt] ? o : n_out - 1;
     }
@@ -105,9 +110,14 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             }
     constexpr int KPG = G / 64 > 0 ? G / 64 : 1; // K iterations per group
     auto load_group_scales = [&](int g, int buf) {
-        const int o = rb * 256 + tid;
-        gsc[buf][tid] = o < n_out ? M.scales[(size_t)o * groups + g] : 0.f;
+        const int o = rb * 128 + tid;
+        if (tid < 128) gsc[buf][tid] = o < n_out ? M.scales[(size_t)o * groups + g] : 0.f;
     };
+    // this block's slice of K, in whole groups
+    const int ks = blockIdx.z;
+    const int n_grp = n_k / KPG;
+    const int kit0 = (int)((long)n_grp * ks / KS) * KPG;
+    const int kit1 = (int)((long)n_grp * (ks + 1) / KS) * KPG;
 
     // staging map: thread -> (token, 16-byte segment) x (TN*8/256) pieces
     constexpr int PIECES = TN * 8 / 256;
@@ -144,14 +154,14 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
         }
     };
 
-    load_stage(0);
-    load_w(0);
+    load_stage(kit0);
+    load_w(kit0);
     store_stage(0);
-    if (SA) load_group_scales(0, 0);
+    if (SA) load_group_scales(kit0 / KPG, (kit0 / KPG) & 1);
     __syncthreads();
 
-    for (int kit = 0; kit < n_k; kit++) {
-        const int buf = kit & 1;
+    for (int kit = kit0; kit < kit1; kit++) {
+        const int buf = (kit - kit0) & 1;
         // this iteration's weights -> registers of their own, then request the next
         uint4 wc[MT];
         h2 noff[MT], s16[MT];
@@ -164,7 +174,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             const _Float16 s = (_Float16)sc[mt];
             s16[mt] = h2{s, s};
         }
-        if (kit + 1 < n_k) {
+        if (kit + 1 < kit1) {
             load_stage(kit + 1);
             load_w(kit + 1);
         }
@@ -196,7 +206,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][wave * 64 + mt * 32 + q * 8 + h * 4]);
+                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][wave * 32 + mt * 32 + q * 8 + h * 4]);
                     const float svv[4] = {sv.x, sv.y, sv.z, sv.w};
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++)
@@ -206,29 +216,37 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                             accg[mt][nb][4 * q + e] = 0.f;
                         }
                 }
-            if (kit + 1 < n_k) load_group_scales((kit + 1) / KPG, gb ^ 1);
+            if (kit + 1 < kit1) load_group_scales((kit + 1) / KPG, gb ^ 1);
         }
-        if (kit + 1 < n_k) store_stage(buf ^ 1);
+        if (kit + 1 < kit1) store_stage(buf ^ 1);
         __syncthreads();
     }
 
     // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4
     const Q4Epi &E = L.e;
+    // workspace of matrix mi starts after those of the matrices before it
+    size_t ws_base = 0;
+    for (int i = 0; i < mi; i++) ws_base += (size_t)KS * B * L.m[i].out;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-        const int obase = (rb * 4 + wave) * (32 * MT) + mt * 32;
+        const int obase = rb * 128 + wave * 32 + mt * 32;
         if (obase >= n_out) continue;
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
             const int t = t0 + nb * 32 + r;
             if (t >= B) continue;
-            const float scale_t = ss ? ss[t] : 1.0f;
             const size_t row = (size_t)t * n_out;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int o = obase + q * 8 + h * 4;
-                float4 v = make_float4(acc[mt][nb][4 * q + 0] * scale_t, acc[mt][nb][4 * q + 1] * scale_t,
-                                       acc[mt][nb][4 * q + 2] * scale_t, acc[mt][nb][4 * q + 3] * scale_t);
+                float4 v = make_float4(acc[mt][nb][4 * q + 0], acc[mt][nb][4 * q + 1], acc[mt][nb][4 * q + 2],
+                                       acc[mt][nb][4 * q + 3]);
+                if (KS > 1) { // partial tile of this K slice
+                    *reinterpret_cast<float4 *>(ws + ws_base + ((size_t)ks * B + t) * n_out + o) = v;
+                    continue;
+                }
+                const float scale_t = ss ? ss[t] : 1.0f;
+                v.x *= scale_t, v.y *= scale_t, v.z *= scale_t, v.w *= scale_t;
                 if (E.kind == Q4_EPI_RESIDUAL) {
                     const float4 rr = *reinterpret_cast<const float4 *>(E.res + row + o);
                     v.x += rr.x;
@@ -244,6 +262,32 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             }
         }
     }
+}
+
+// Adds the KS partial tiles of a split-K GEMM in slice order and runs the epilogue.
+// grid: (ceil(sum_out / 256), B); the matrices of the launch are laid end to end.
+__global__ __launch_bounds__(256) void q4_gemm_reduce_kernel(const Q4Launch L, const float *__restrict__ ss,
+                                                             const float *__restrict__ ws, int KS) {
+    const int t = blockIdx.y;
+    int o = blockIdx.x * 256 + threadIdx.x;
+    int mi = 0;
+    size_t ws_base = 0;
+    const int B = L.batch;
+    while (mi + 1 < L.n_mats && o >= L.m[mi].out) {
+        o -= L.m[mi].out;
+        ws_base += (size_t)KS * B * L.m[mi].out;
+        mi++;
+    }
+    const Q4Mat &M = L.m[mi];
+    if (o >= M.out) return;
+    float v = 0.f;
+    for (int ks = 0; ks < KS; ks++) v += ws[ws_base + ((size_t)ks * B + t) * M.out + o];
+    if (ss) v *= ss[t];
+    const Q4Epi &E = L.e;
+    const size_t row = (size_t)t * M.out;
+    if (E.kind == Q4_EPI_RESIDUAL) v += E.res[row + o];
+    if (E.kind != Q4_EPI_SCATTER_ONLY) M.y[row + o] = v;
+    for (int c = 0; c < E.n_scatter; c++) E.sc_out[c][row + E.sc_idx[c][o]] = v;
 }
 
 // fp32 [B][n] (already in the consumer's g_index order) -> fp16 [B][n], times the
@@ -302,38 +346,53 @@ __global__ void silu_scatter_kernel(float *out, const float *a, const float *c, 
 }
 
 template <int G>
-int launch_gemm_g(Q4Launch &L, const XhList &xh_list_dev, const float *ss, hipStream_t st) {
+int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st) {
     int total = 0;
+    long rows = 0;
     for (int i = 0; i < L.n_mats; i++) {
-        L.m[i].row_blocks = (L.m[i].out + 255) / 256;
+        L.m[i].row_blocks = (L.m[i].out + 127) / 128;
         total += L.m[i].row_blocks;
+        rows += L.m[i].out;
     }
     const int B = L.batch;
     const int NB = B > 64 ? 4 : B > 32 ? 2 : 1;
     const int TN = 32 * NB;
-    dim3 grid(total, (B + TN - 1) / TN), block(256);
+    const int t_tiles = (B + TN - 1) / TN;
+    // K slices: aim at ~2 blocks per CU, whole groups per slice, at most 8
+    const int n_grp = (L.in / 64) / (G / 64 > 0 ? G / 64 : 1);
+    int KS = (512 + total * t_tiles - 1) / (total * t_tiles);
+    if (KS > 8) KS = 8;
+    if (KS > n_grp) KS = n_grp;
+    if (KS < 1) KS = 1;
+    while (KS > 1 && (size_t)KS * B * rows > ws_floats) KS--;
+    dim3 grid(total, t_tiles, KS), block(256);
     const size_t lds = (size_t)2 * TN * kXRow * sizeof(_Float16);
     switch (NB) {
-        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1>), grid, block, lds, st, L, xh_list_dev, ss); break;
-        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2>), grid, block, lds, st, L, xh_list_dev, ss); break;
-        default: hipLaunchKernelGGL((q4_gemm_kernel<G, 4>), grid, block, lds, st, L, xh_list_dev, ss); break;
+        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1>), grid, block, lds, st, L, xh, ss, ws, KS); break;
+        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2>), grid, block, lds, st, L, xh, ss, ws, KS); break;
+        default: hipLaunchKernelGGL((q4_gemm_kernel<G, 4>), grid, block, lds, st, L, xh, ss, ws, KS); break;
     }
     L2_HIP(hipGetLastError());
+    if (KS > 1) {
+        hipLaunchKernelGGL(q4_gemm_reduce_kernel, dim3((unsigned)((rows + 255) / 256), B), dim3(256), 0, st, L, ss, ws, KS);
+        L2_HIP(hipGetLastError());
+    }
     return L2_OK;
 }
 
 } // namespace
 
-int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, hipStream_t st) {
+int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, float *ws, size_t ws_floats,
+                   hipStream_t st) {
     if (L.n_mats < 1 || L.n_mats > 3) return l2_fail(L2_ERR_ARG, "q4 gemm: n_mats=%d", L.n_mats);
     if (L.in % 64 != 0 || L.in % L.group_size != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d must be a multiple of 64", L.in);
     for (int i = 0; i < L.n_mats; i++)
         if (L.m[i].out % 32 != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: out=%d must be a multiple of 32", L.m[i].out);
     if (L.pair) return l2_fail(L2_ERR_ARG, "q4 gemm: pair launches are not supported");
     switch (L.group_size) {
-        case 32: return launch_gemm_g<32>(L, xh_list_dev, ss, st);
-        case 64: return launch_gemm_g<64>(L, xh_list_dev, ss, st);
-        case 128: return launch_gemm_g<128>(L, xh_list_dev, ss, st);
+        case 32: return launch_gemm_g<32>(L, xh_list_dev, ss, ws, ws_floats, st);
+        case 64: return launch_gemm_g<64>(L, xh_list_dev, ss, ws, ws_floats, st);
+        case 128: return launch_gemm_g<128>(L, xh_list_dev, ss, ws, ws_floats, st);
     }
     return l2_fail(L2_ERR_ARG, "q4 gemm: group size %d", L.group_size);
 }

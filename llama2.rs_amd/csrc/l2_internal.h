@@ -105,8 +105,9 @@ struct XhList {
     const void *p[3]; // per matrix of the launch: fp16 [B][in], g_index order, pair-interleaved (prep_f16_launch)
 };
 // Y = X W^T for a chunk of L.batch tokens; ss (per token, may be null) scales the rows of Y.
-// Epilogues as in the matvec (no pair launches).
-int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, hipStream_t st);
+// Epilogues as in the matvec (no pair launches).  ws: workspace of ws_floats floats for split-K partial
+// tiles (the launcher uses as many K slices as fit).
+int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st);
 bool q4_gemm_supports(int in, int out);
 // out_f16[b][j'] = fp16(x[b][j] * (wn ? wn[j] : 1)), j' = j with the order (0,4,1,5,2,6,3,7) inside every 8.
 int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st);
