@@ -14,11 +14,122 @@
 // row); those go to a small double-buffered LDS tile [row][NWK*4]; after one
 // barrier per tile of P*S rows, one thread per row adds them in a fixed order
 // and runs the epilogue.  No atomics: results are bit-stable.
+//
+// Integer form (IDOT).  The vector ALU is the co-bottleneck of the fp32 form
+// (one FMA, one convert-equivalent and 3/8 of a mask per nibble), so the default
+// form keeps the arithmetic in integers: after staging, the block quantises x
+// once, chunk by chunk, to 24-bit fixed point against a power-of-two step
+// (delta = 2^(e-22), |x| < 2^e within the chunk) and stores it as six planes of
+// balanced base-16 digits (-8..7), 8 digits per word in the nibble order of the
+// weights.  A weight word XOR 0x88888888 is the 8 signed nibbles n - 8, so
+// v_dot8_i32_i4 multiplies one weight word with one digit word: 24 instructions
+// per 32 weights instead of ~76, exact integer sums, and
+//   sum_k (n_k - z1) x_k = delta * (I - (z1 - 8) * sum_k q_k),  I = sum_d 16^d a_d.
+// The quantisation error (2^-23 of the chunk maximum per element) is of the
+// size of fp32 rounding.
+#include <string.h>
+
 #include "q4_common.h"
 
 namespace {
 
 using namespace q4;
+
+constexpr int kPlaneWords = 28; // per chunk: 6 planes x 4 words, delta, sum of q, 2 pad
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_xchg_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+
+// Quantise a staged vector (xs[c*36 + i], c < C, i < 32) in place into digit
+// planes: word (c, d, j) at ((uint32_t*)xs)[c*28 + d*4 + j]; delta and sum(q)
+// as floats at [c*28 + 24], [c*28 + 25].  Thread -> (chunk, word of 8 elements);
+// the 4 threads of a chunk are adjacent lanes.  Outputs only ever land on
+// inputs of lower chunks, which are consumed in earlier passes.
+template <int NT>
+__device__ __forceinline__ void quantize_in_place(float *xs, int C, int tid) {
+    uint32_t *xw = reinterpret_cast<uint32_t *>(xs);
+    const int n_words = C * 4;
+    for (int base = 0; base < n_words; base += NT) {
+        const int wi = base + tid;
+        const bool ok = wi < n_words;
+        const int c = wi >> 2, j = wi & 3;
+        float v[8];
+        if (ok) {
+            const float4 a = *reinterpret_cast<const float4 *>(&xs[c * kChunkPad + j * 8]);
+            const float4 b = *reinterpret_cast<const float4 *>(&xs[c * kChunkPad + j * 8 + 4]);
+            v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = 0.f;
+        }
+        float am = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) am = fmaxf(am, fabsf(v[e]));
+        am = fmaxf(am, dpp_xchg<0xB1>(am));
+        am = fmaxf(am, dpp_xchg<0x4E>(am));
+        // am < 2^(eb-126): step 2^(eb-148) keeps |x/step| < 2^22
+        int eb = (int)((__builtin_bit_cast(uint32_t, am) >> 23) & 0xFFu);
+        eb = eb < 22 ? 22 : eb;
+        const float inv = __builtin_bit_cast(float, (uint32_t)(275 - eb) << 23);
+        const float delta = __builtin_bit_cast(float, (uint32_t)(eb - 21) << 23);
+        uint32_t u[8];
+        int sq = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int q = (int)rintf(v[e] * inv);
+            sq += q;
+            u[e] = (uint32_t)(q + 0x888888);
+        }
+        sq += dpp_xchg_i<0xB1>(sq);
+        sq += dpp_xchg_i<0x4E>(sq);
+        uint32_t pw[6];
+#pragma unroll
+        for (int d = 0; d < 6; d++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 8; e++) w |= ((u[e] >> (4 * d)) & 15u) << (4 * e);
+            pw[d] = w ^ 0x88888888u; // unsigned digit - 8 as a signed nibble
+        }
+        __syncthreads(); // every input of this pass is in registers
+        if (ok) {
+#pragma unroll
+            for (int d = 0; d < 6; d++) xw[c * kPlaneWords + d * 4 + j] = pw[d];
+            if (j == 0) {
+                xs[c * kPlaneWords + 24] = delta;
+                xs[c * kPlaneWords + 25] = (float)sq;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// sum_k (n_k - 8) q_k over one chunk: 4 weight words against 6 digit planes.
+__device__ __forceinline__ float chunk_idot(const uint4 w, const int (&xp)[24]) {
+    const int w0 = (int)(w.x ^ 0x88888888u), w1 = (int)(w.y ^ 0x88888888u), w2 = (int)(w.z ^ 0x88888888u),
+              w3 = (int)(w.w ^ 0x88888888u);
+    int a[6];
+#pragma unroll
+    for (int d = 0; d < 6; d++) {
+        int t = __builtin_amdgcn_sdot8(w0, xp[d * 4 + 0], 0, false);
+        t = __builtin_amdgcn_sdot8(w1, xp[d * 4 + 1], t, false);
+        t = __builtin_amdgcn_sdot8(w2, xp[d * 4 + 2], t, false);
+        a[d] = __builtin_amdgcn_sdot8(w3, xp[d * 4 + 3], t, false);
+    }
+    const int lo = (((a[2] << 4) + a[1]) << 4) + a[0];
+    const int hi = (((a[5] << 4) + a[4]) << 4) + a[3];
+    return fmaf((float)hi, 4096.0f, (float)lo);
+}
+
+template <class T>
+__device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_offset);
+}
+
+__device__ __forceinline__ void st_at(float *base, uint32_t byte_offset, float v) {
+    *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + byte_offset) = v;
+}
 
 struct RowData {
     uint4 w;
@@ -26,7 +137,7 @@ struct RowData {
     int32_t z;
 };
 
-template <int G, int NWK, int S, bool PAIR>
+template <int G, int NWK, int S, bool PAIR, bool IDOT>
 __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L) {
     constexpr int NM = PAIR ? 2 : 1;
     constexpr int NW = NWK * S;
@@ -65,26 +176,32 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     const int row1 = min(row0 + L.rows_per_block, n_out);
     const int c = kslice * 64 + lane; // this lane's chunk, for good
     const bool has_chunk = c < C;
-    const int g = has_chunk ? c / CPG : 0;
 
-    // row i of this stream is row0 + stream + i * S
-    auto fetch = [&](int i, RowData(&d)[NM]) {
-        const int o = row0 + stream + i * S;
-        if (has_chunk && o < row1) {
+    // Row i of this stream is row0 + stream + i * S. Loads are unconditional so
+    // that the loop body stays one basic block and every wait names only the
+    // oldest row in flight: rows past the end re-read the block's last row and
+    // lanes past the last chunk re-read the last chunk (their x is zero).
+    const int cc = has_chunk ? c : C - 1;
+    const int g = cc / CPG;
+    const int last = row1 - 1;
+    const uint4 *__restrict__ wq[NM];
+    const float *__restrict__ sc[NM];
+    const int32_t *__restrict__ zq[NM];
 #pragma unroll
-            for (int q = 0; q < NM; q++) {
-                const Q4Mat &M = L.m[mi + q];
-                d[q].w = M.qweight[(size_t)o * C + c];
-#ifdef L2_Q4_DEBUG
-                if (L.e.kind >= 103) { // weights only
-                    d[q].s = 1.f;
-                    d[q].z = 0;
-                    continue;
-                }
-#endif
-                d[q].s = M.scales[(size_t)o * groups + g];
-                d[q].z = M.qzeros[(size_t)(o >> 3) * groups + g];
-            }
+    for (int q = 0; q < NM; q++) {
+        wq[q] = L.m[mi + q].qweight;
+        sc[q] = L.m[mi + q].scales;
+        zq[q] = L.m[mi + q].qzeros;
+    }
+    auto fetch = [&](int i, RowData(&d)[NM]) {
+        const int o = min(row0 + stream + i * S, last);
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            // 24-bit multiplies and 32-bit byte offsets from a uniform base:
+            // no 64-bit address arithmetic per load
+            d[q].w = ld_at<uint4>(wq[q], (__umul24(o, C) + cc) << 4);
+            d[q].s = ld_at<float>(sc[q], (__umul24(o, groups) + g) << 2);
+            d[q].z = ld_at<int32_t>(zq[q], (__umul24(o >> 3, groups) + g) << 2);
         }
     };
 
@@ -117,33 +234,93 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         t += L.eps;
         ss = 1.0f / sqrtf(t);
     }
-    float x[NM][32];
-    float sx[NM];
+    // this lane's slice of x, for good: 32 floats, or 24 digit words + step + sum of q
+    float x[NM][IDOT ? 1 : 32];
+    int xp[NM][IDOT ? 24 : 1];
+    float sx[NM];     // fp32 form: sum of the chunk's x; integer form: sum of its q
+    float xdelta[NM]; // integer form: the chunk's step
+    if constexpr (IDOT) {
+#pragma unroll
+        for (int q = 0; q < NM; q++) quantize_in_place<NW * 64>(lds + q * xstride, C, tid);
+    }
 #pragma unroll
     for (int q = 0; q < NM; q++) {
         const float *xs = lds + q * xstride;
-        if (has_chunk) {
-            const float4 *p = reinterpret_cast<const float4 *>(&xs[c * kChunkPad]);
+        xdelta[q] = 0.f;
+        sx[q] = 0.f;
+        if constexpr (IDOT) {
+            if (has_chunk) {
+                const uint4 *p = reinterpret_cast<const uint4 *>(&xs[c * kPlaneWords]);
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float4 v = p[i];
-                x[q][4 * i + 0] = v.x;
-                x[q][4 * i + 1] = v.y;
-                x[q][4 * i + 2] = v.z;
-                x[q][4 * i + 3] = v.w;
+                for (int i = 0; i < 6; i++) {
+                    const uint4 v = p[i];
+                    xp[q][4 * i + 0] = (int)v.x;
+                    xp[q][4 * i + 1] = (int)v.y;
+                    xp[q][4 * i + 2] = (int)v.z;
+                    xp[q][4 * i + 3] = (int)v.w;
+                }
+                xdelta[q] = xs[c * kPlaneWords + 24];
+                sx[q] = xs[c * kPlaneWords + 25];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 24; i++) xp[q][i] = 0;
             }
-            sx[q] = xs[C * kChunkPad + c];
         } else {
+            if (has_chunk) {
+                const float4 *p = reinterpret_cast<const float4 *>(&xs[c * kChunkPad]);
 #pragma unroll
-            for (int i = 0; i < 32; i++) x[q][i] = 0.f;
-            sx[q] = 0.f;
+                for (int i = 0; i < 8; i++) {
+                    const float4 v = p[i];
+                    x[q][4 * i + 0] = v.x;
+                    x[q][4 * i + 1] = v.y;
+                    x[q][4 * i + 2] = v.z;
+                    x[q][4 * i + 3] = v.w;
+                }
+                sx[q] = xs[C * kChunkPad + c];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 32; i++) x[q][i] = 0.f;
+            }
         }
     }
 
     const int n_rows = row1 - row0;
     const int n_tiles = (n_rows + TR - 1) / TR;
     int buf = 0;
+    // Enter the loop with no load outstanding (the primed rows arrived while x
+    // was staged). The compiler's wait counts inside the loop are then those of
+    // the steady state alone: vmcnt leaves the P - 1 younger rows in flight.
+    // Otherwise the issue order of the prologue leaks into the loop's waits.
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0), expcnt and lgkmcnt untouched
+    // Epilogue operands, uniform for the block.
+    const Q4Epi &E = L.e;
+    const int epi_kind = E.kind;
+    const int n_scatter = E.n_scatter;
+    const size_t out_base = (size_t)b * n_out;
+    const float *__restrict__ res = E.res;
+    float *__restrict__ const yout = L.m[mi].y;
+    const int32_t *__restrict__ sc_idx[3] = {E.sc_idx[0], E.sc_idx[1], E.sc_idx[2]};
+    float *__restrict__ sc_out[3] = {E.sc_out[0], E.sc_out[1], E.sc_out[2]};
+    // what the epilogue lanes prefetch; the scales (at least one word per row) stand in for absent operands
+    const bool has_res = !PAIR && epi_kind == Q4_EPI_RESIDUAL;
+    const float *__restrict__ res_p = has_res ? res + out_base : sc[0];
+    const int32_t *__restrict__ idx_p[3];
+#pragma unroll
+    for (int t = 0; t < 3; t++) idx_p[t] = t < n_scatter ? sc_idx[t] : reinterpret_cast<const int32_t *>(sc[0]);
+
     for (int tile = 0; tile < n_tiles; tile++) {
+        // The lanes that finish this tile's rows fetch what the epilogue reads
+        // (residual, scatter indices) now: by the time it is needed, P rows of
+        // younger loads stand behind it and the wait leaves those in flight.
+        const int eo = row0 + tile * TR + tid;
+        const bool epi = tid < TR && eo < row1;
+        float res_v = 0.f;
+        uint32_t sidx[3] = {0, 0, 0};
+        if (epi) { // no branch per operand: an unused one reads a valid dummy
+            res_v = res_p[eo];
+#pragma unroll
+            for (int t = 0; t < 3; t++) sidx[t] = (uint32_t)idx_p[t][eo];
+        }
 #pragma unroll
         for (int u = 0; u < P; u++) {
             const int i = tile * P + u;
@@ -151,22 +328,26 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
             float pr[NM];
 #pragma unroll
             for (int q = 0; q < NM; q++) {
-                float v = 0.f;
-                if (has_chunk && o < row1) {
-#ifdef L2_Q4_DEBUG
-                    const uint4 ww = pipe[u][q].w;
-                    const float p = (L.e.kind >= 101) ? __builtin_bit_cast(float, (ww.x ^ ww.y ^ ww.z ^ ww.w) & 0x3fffffffu) + x[q][u]
-                                                      : chunk_dot(ww, x[q]);
-#else
+                const int zn = (pipe[u][q].z >> (4 * (o & 7))) & 15;
+                if constexpr (IDOT) {
+                    const float f = chunk_idot(pipe[u][q].w, xp[q]);
+                    pr[q] = (pipe[u][q].s * xdelta[q]) * fmaf(-(float)(zn - 7), sx[q], f);
+                } else {
                     const float p = chunk_dot(pipe[u][q].w, x[q]);
-#endif
-                    const int zn = (pipe[u][q].z >> (4 * (o & 7))) & 15;
                     const float z1 = (float)(zn + 1);
-                    v = pipe[u][q].s * fmaf(p, 512.0f, -z1 * sx[q]);
+                    pr[q] = pipe[u][q].s * fmaf(p, 512.0f, -z1 * sx[q]);
                 }
-                pr[q] = v;
             }
-            fetch(i + P, pipe[u]); // refill this slot: row i + P
+            // Refill this slot with row i + P, after its last use and not before:
+            // a load hoisted above the row's arithmetic makes the compiler copy
+            // live registers of the other slots, and each copy waits on its load.
+            // The empty statements pin the row's result before the loads and
+            // the loads before what follows.
+            if constexpr (NM == 2) asm volatile("" : "+v"(pr[0]), "+v"(pr[NM - 1])::"memory");
+            else asm volatile("" : "+v"(pr[0])::"memory");
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(i + P, pipe[u]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int q = 0; q < NM; q++) {
                 float v = pr[q];
@@ -177,34 +358,28 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
                 if ((lane & 15) == 0) part[buf][u * S + stream][q][kslice * 4 + (lane >> 4)] = v;
             }
         }
-#ifdef L2_Q4_DEBUG
-        if (L.e.kind == 104) continue; // no reduction barrier, no epilogue
-#endif
         __syncthreads();
-        if (tid < TR) {
-            const int o = row0 + tile * TR + tid;
-            if (o < row1) {
-                float sum[NM];
+        if (epi) {
+            float sum[NM];
 #pragma unroll
-                for (int q = 0; q < NM; q++) {
-                    float a = 0.f;
+            for (int q = 0; q < NM; q++) {
+                float a = 0.f;
 #pragma unroll
-                    for (int k = 0; k < PW; k++) a += part[buf][tid][q][k];
-                    sum[q] = a;
-                }
-                const Q4Epi &E = L.e;
-                const size_t row = (size_t)b * n_out;
-                float v = sum[0] * ss;
-                if (PAIR) { // silu(w1 x) * (w3 x), src/models.rs:92-98
-                    const float u2 = sum[NM - 1] * ss;
-                    v = v * (1.0f / (1.0f + expf(-v)));
-                    v = v * u2;
-                } else if (E.kind == Q4_EPI_RESIDUAL) {
-                    v = E.res[row + o] + v;
-                }
-                if (E.kind != Q4_EPI_SCATTER_ONLY) L.m[mi].y[row + o] = v;
-                for (int t = 0; t < E.n_scatter; t++) E.sc_out[t][row + E.sc_idx[t][o]] = v;
+                for (int k = 0; k < PW; k++) a += part[buf][tid][q][k];
+                sum[q] = a;
             }
+            float v = sum[0] * ss;
+            if (PAIR) { // silu(w1 x) * (w3 x), src/models.rs:92-98
+                const float u2 = sum[NM - 1] * ss;
+                v = v * (1.0f / (1.0f + expf(-v)));
+                v = v * u2;
+            } else if (epi_kind == Q4_EPI_RESIDUAL) {
+                v = res_v + v;
+            }
+            if (epi_kind != Q4_EPI_SCATTER_ONLY) yout[out_base + eo] = v;
+#pragma unroll
+            for (int t = 0; t < 3; t++)
+                if (t < n_scatter) st_at(sc_out[t], ((uint32_t)out_base + sidx[t]) << 2, v); // 32-bit offset: nothing widens the loaded index
         }
         buf ^= 1;
     }
@@ -222,7 +397,7 @@ int cu_count() {
     return n;
 }
 
-template <int G, int NWK, int S, bool PAIR>
+template <int G, int NWK, int S, bool PAIR, bool IDOT>
 int launch_s(Q4Launch &L, hipStream_t stream) {
     constexpr int NW = NWK * S;
     constexpr int TR = (PAIR ? Q4S_P / 2 : Q4S_P) * S;
@@ -249,7 +424,7 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     }
     L.rows_per_block = rpb;
     for (int i = 0; i < L.n_mats; i++) L.m[i].row_blocks = (L.m[i].out + rpb - 1) / rpb;
-    auto kern = q4_stream_kernel<G, NWK, S, PAIR>;
+    auto kern = q4_stream_kernel<G, NWK, S, PAIR, IDOT>;
     if (lds > 48 * 1024) {
         static size_t raised = 0; // per instantiation
         if (lds > raised) {
@@ -269,26 +444,26 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     return L2_OK;
 }
 
-template <int G>
+template <int G, bool IDOT>
 int launch_sg(Q4Launch &L, hipStream_t stream) {
     const int nwk = (L.in / 32 + 63) / 64;
     if (!L.pair) {
         switch (nwk) {
-            case 1: return launch_s<G, 1, 4, false>(L, stream);
-            case 2: return launch_s<G, 2, 4, false>(L, stream);
-            case 3: return launch_s<G, 3, 4, false>(L, stream);
-            case 4: return launch_s<G, 4, 4, false>(L, stream);
-            case 5: case 6: return launch_s<G, 6, 2, false>(L, stream);
-            case 7: return launch_s<G, 7, 2, false>(L, stream);
-            case 8: return launch_s<G, 8, 2, false>(L, stream);
-            case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false>(L, stream);
+            case 1: return launch_s<G, 1, 4, false, IDOT>(L, stream);
+            case 2: return launch_s<G, 2, 4, false, IDOT>(L, stream);
+            case 3: return launch_s<G, 3, 4, false, IDOT>(L, stream);
+            case 4: return launch_s<G, 4, 4, false, IDOT>(L, stream);
+            case 5: case 6: return launch_s<G, 6, 2, false, IDOT>(L, stream);
+            case 7: return launch_s<G, 7, 2, false, IDOT>(L, stream);
+            case 8: return launch_s<G, 8, 2, false, IDOT>(L, stream);
+            case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, IDOT>(L, stream);
         }
     } else {
         switch (nwk) {
-            case 1: return launch_s<G, 1, 4, true>(L, stream);
-            case 2: return launch_s<G, 2, 4, true>(L, stream);
-            case 3: return launch_s<G, 3, 2, true>(L, stream);
-            case 4: return launch_s<G, 4, 2, true>(L, stream);
+            case 1: return launch_s<G, 1, 4, true, IDOT>(L, stream);
+            case 2: return launch_s<G, 2, 4, true, IDOT>(L, stream);
+            case 3: return launch_s<G, 3, 2, true, IDOT>(L, stream);
+            case 4: return launch_s<G, 4, 2, true, IDOT>(L, stream);
         }
     }
     return l2_fail(L2_ERR_ARG, "q4 matvec (streaming): in=%d pair=%d has no kernel", L.in, L.pair);
@@ -297,14 +472,23 @@ int launch_sg(Q4Launch &L, hipStream_t stream) {
 } // namespace
 
 int q4_stream_launch(Q4Launch &L, hipStream_t stream) {
-#ifdef L2_Q4_DEBUG
-    static const int dbg = getenv("L2_Q4_DBG") ? atoi(getenv("L2_Q4_DBG")) : 0;
-    if (dbg) L.e.kind = dbg;
-#endif
-    switch (L.group_size) {
-        case 32: return launch_sg<32>(L, stream);
-        case 64: return launch_sg<64>(L, stream);
-        case 128: return launch_sg<128>(L, stream);
+    // L2_Q4_IMPL=idot selects the integer-dot form of the inner loop; the default is the fp32 form.
+    static const bool fp32_form = []() {
+        const char *v = getenv("L2_Q4_IMPL");
+        return !(v && !strcmp(v, "idot"));
+    }();
+    if (fp32_form) {
+        switch (L.group_size) {
+            case 32: return launch_sg<32, false>(L, stream);
+            case 64: return launch_sg<64, false>(L, stream);
+            case 128: return launch_sg<128, false>(L, stream);
+        }
+    } else {
+        switch (L.group_size) {
+            case 32: return launch_sg<32, true>(L, stream);
+            case 64: return launch_sg<64, true>(L, stream);
+            case 128: return launch_sg<128, true>(L, stream);
+        }
     }
     return l2_fail(L2_ERR_ARG, "q4 matvec: group size %d (32, 64 or 128)", L.group_size);
 }
