@@ -28,6 +28,7 @@ SOURCES = {
     "kernels_q4_gemm.hip": [],
     # the block kernels keep the reference's rounded-multiply-then-add where they restate it
     "kernels_misc.hip": ["-ffp-contract=off"],
+    "kernels_attn.hip": ["-ffp-contract=off"],
     "host.cpp": ["-x", "hip", "-ffp-contract=off"],
     "textgen.cpp": ["-x", "hip", "-ffp-contract=off"],
 }

@@ -955,12 +955,10 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
                 a.ts = 256;
                 a.n_splits = 1;
             } else {
-                // enough blocks to cover the CUs, at least 64 timesteps each
-                int want = (256 + d.n_kv_heads - 1) / d.n_kv_heads;
+                // two blocks per CU where the context allows it, at least 64 timesteps each
+                int want = (512 + d.n_kv_heads - 1) / d.n_kv_heads;
                 if (want > kMaxSplits) want = kMaxSplits;
                 int ts = ((n_t + want - 1) / want + 63) / 64 * 64;
-                const int qg = d.n_heads / d.n_kv_heads;
-                while ((size_t)ts * qg * 4 > 32 * 1024) ts -= 64;
                 if (ts < 64) ts = 64;
                 a.ts = ts;
                 a.n_splits = (n_t + ts - 1) / ts;

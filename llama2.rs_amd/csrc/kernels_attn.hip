@@ -1,0 +1,362 @@
+// Decode attention for one query position (src/models.rs:131-176, :228-256):
+// RoPE on q and on the new key, the cache write, scores, softmax and the
+// weighted sum of values in one kernel; a second, small kernel merges the
+// splits when the timesteps are cut across several blocks.  gfx950, wave64.
+//
+// The softmax is computed in the running-maximum form: every group of lanes
+// keeps (m, l, acc) = (largest score so far, sum of e^(s - m), sum of
+// e^(s - m) v) and rescales when m grows; groups, waves and splits are merged
+// by the same rule.  That is the function softmax(src/util.rs:49-65) followed
+// by the weighted sum (:160-174); only the order of the roundings differs.
+// Scores are kept in units of log2: t = (q.k) * log2(e) / sqrt(head_size), so
+// that e^(s - m) is one v_exp_f32 of t - m (1 ulp; the scaling of the argument
+// adds a relative error of about |s - m| * 6e-8 to a weight).
+//
+// Compiled with -ffp-contract=off; FMAs appear only where written as fmaf().
+#include "l2_internal.h"
+
+namespace {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_xchg(float v) {
+    int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+    return __builtin_bit_cast(float, r);
+}
+
+template <class T>
+__device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_offset);
+}
+
+constexpr float kNoScore = -1e30f; // "no timestep yet": finite, so that differences never give NaN
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_xchg<0xB1>(v);
+    v += dpp_xchg<0x4E>(v);
+    v += dpp_xchg<0x141>(v);
+    v += dpp_xchg<0x140>(v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_xchg<0xB1>(v));
+    v = fmaxf(v, dpp_xchg<0x4E>(v));
+    v = fmaxf(v, dpp_xchg<0x141>(v));
+    v = fmaxf(v, dpp_xchg<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+
+// Layout of a block: 4 waves x 4 rows of 16 lanes.  One row of lanes handles
+// one timestep at a time, each lane 8 of the 128 head dimensions; a block
+// covers 16 timesteps per step and PD steps per tile, all of a tile's loads
+// being issued before its arithmetic.  All QG query heads of the kv head share
+// each K and V load (grouped-query attention, src/models.rs:142-145).
+template <int QG>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
+    constexpr int HS = 128, HALF = 64;
+    constexpr int PD = QG >= 8 ? 2 : 4;
+    __shared__ float qs[QG * HS];
+    __shared__ float kvnew[2][HS];
+    __shared__ float comb[4][QG][HS + 2];
+    const int kvh = blockIdx.x, sp = blockIdx.y;
+    const int pos = A.dpos[0];
+    const int t0 = sp * A.ts;
+    if (t0 > pos) return;
+    const int t1 = min(t0 + A.ts, pos + 1);
+    const int n = t1 - t0;
+    const int kv_dim = A.n_kv_heads * HS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ds = lane & 15;            // dims [8 ds, 8 ds + 8)
+    const int tl = wave * 4 + (lane >> 4); // this row's timestep within a step of 16
+
+    const float *__restrict__ kc = A.kcache;
+    const float *__restrict__ vc = A.vcache;
+    const uint32_t row_bytes = (uint32_t)kv_dim * 4u;
+    const uint32_t lane_off = (uint32_t)(kvh * HS + ds * 8) * 4u;
+    const int t_last = t1 - 1;
+
+    struct Step {
+        float4 k0, k1, v0, v1;
+    };
+    // Unconditional loads: rows past the end re-read the last row, and the row
+    // of the new position is read although its values are replaced below.
+    auto fetch = [&](int it, Step &d) {
+        const int t = min(t0 + it * 16 + tl, t_last);
+        const uint32_t off = __umul24(t, row_bytes) + lane_off;
+        d.k0 = ld_at<float4>(kc, off);
+        d.k1 = ld_at<float4>(kc, off + 16);
+        d.v0 = ld_at<float4>(vc, off);
+        d.v1 = ld_at<float4>(vc, off + 16);
+    };
+    // The small loads that the staging below needs go out first: loads return in
+    // order, so behind the first tile's loads they would wait for all of them.
+    // Every thread stages something (threads beyond the work repeat another
+    // thread's element), so that no load can move into a branch further down.
+    const float *ct = A.cos_t + (size_t)pos * HALF;
+    const float *st = A.sin_t + (size_t)pos * HALF;
+    constexpr int NQ = (QG * HALF + 255) / 256;
+    float qa[NQ], qb[NQ], qc[NQ], qsn[NQ];
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const int idx = (tid + r * 256) % (QG * HALF);
+        const int j = idx >> 6, i = idx & 63;
+        const float *qh = A.q + (size_t)(kvh * QG + j) * HS;
+        qa[r] = qh[i], qb[r] = qh[i + HALF];
+        qc[r] = ct[i], qsn[r] = st[i];
+    }
+    const int hd = tid & 63;
+    const float nk_a = A.k_new[(size_t)kvh * HS + hd], nk_b = A.k_new[(size_t)kvh * HS + hd + HALF];
+    const float nv = A.v_new[(size_t)kvh * HS + (tid & 127)];
+    const float nc = ct[hd], ns = st[hd];
+    __builtin_amdgcn_sched_barrier(0);
+
+    Step pipe[PD];
+#pragma unroll
+    for (int u = 0; u < PD; u++) fetch(u, pipe[u]); // first tile: in flight while q is staged
+    __builtin_amdgcn_sched_barrier(0);
+
+    // q with RoPE, src/models.rs:100-129 (the second half uses the rotated first half)
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const int idx = (tid + r * 256) % (QG * HALF);
+        const int j = idx >> 6, i = idx & 63;
+        const float first = qa[r] * qc[r] - qb[r] * qsn[r];
+        qs[j * HS + i] = first;
+        qs[j * HS + HALF + i] = qb[r] * qc[r] + first * qsn[r];
+    }
+    // the new key, rotated, and the new value; the block whose range ends at pos
+    // also writes them to the cache (:236-249)
+    const bool owns_new = (t1 == pos + 1);
+    {
+        const float first = nk_a * nc - nk_b * ns;
+        const float second = nk_b * nc + first * ns;
+        kvnew[0][hd] = first;
+        kvnew[0][hd + HALF] = second;
+        kvnew[1][tid & 127] = nv;
+        if (owns_new) {
+            if (tid < HALF) {
+                float *kw = A.kcache + (size_t)pos * kv_dim + kvh * HS;
+                kw[tid] = first;
+                kw[tid + HALF] = second;
+            } else if (tid >= 128) {
+                A.vcache[(size_t)pos * kv_dim + kvh * HS + (tid - 128)] = nv;
+            }
+        }
+    }
+    __syncthreads();
+
+    // q in registers, except for 8 heads per kv head, where the registers go to the accumulators
+    constexpr bool kQInLds = QG >= 8;
+    float q[kQInLds ? 1 : QG][8];
+    if constexpr (!kQInLds) {
+#pragma unroll
+        for (int j = 0; j < QG; j++) {
+            const float4 a = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8]);
+            const float4 b = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8 + 4]);
+            q[j][0] = a.x, q[j][1] = a.y, q[j][2] = a.z, q[j][3] = a.w;
+            q[j][4] = b.x, q[j][5] = b.y, q[j][6] = b.z, q[j][7] = b.w;
+        }
+    }
+    float m[QG], l[QG], acc[QG][8];
+#pragma unroll
+    for (int j = 0; j < QG; j++) {
+        m[j] = kNoScore;
+        l[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[j][e] = 0.f;
+    }
+    // log2(e) / sqrt(head_size): src/models.rs:154 divides the score by sqrt(head_size)
+    const float scale = 1.44269504088896340736f / sqrtf((float)HS);
+    const int n_it = (n + 15) >> 4;
+    const int n_tiles = (n_it + PD - 1) / PD;
+    for (int tile = 0; tile < n_tiles; tile++) {
+        if (tile > 0) { // all of the tile's loads, then its arithmetic
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < PD; u++) fetch(tile * PD + u, pipe[u]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int u = 0; u < PD; u++) {
+            const int t = t0 + (tile * PD + u) * 16 + tl;
+            const bool valid = t < t1;
+            const Step &d = pipe[u];
+            float k[8] = {d.k0.x, d.k0.y, d.k0.z, d.k0.w, d.k1.x, d.k1.y, d.k1.z, d.k1.w};
+            float v[8] = {d.v0.x, d.v0.y, d.v0.z, d.v0.w, d.v1.x, d.v1.y, d.v1.z, d.v1.w};
+            if (__any(t == pos)) { // once per block: the row of the new position comes from LDS, not from the cache
+                const bool is_new = t == pos;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    k[e] = is_new ? kvnew[0][ds * 8 + e] : k[e];
+                    v[e] = is_new ? kvnew[1][ds * 8 + e] : v[e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = valid ? v[e] : 0.f; // a row past the end may hold anything, NaN included
+            float sc[QG];
+            bool grow = false;
+#pragma unroll
+            for (int j = 0; j < QG; j++) {
+                float s = 0.f;
+                if constexpr (kQInLds) {
+                    const float4 a = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8]);
+                    const float4 b = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8 + 4]);
+                    const float qj[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) s = fmaf(qj[e], k[e], s);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) s = fmaf(q[j][e], k[e], s);
+                }
+                s += dpp_xchg<0xB1>(s);
+                s += dpp_xchg<0x4E>(s);
+                s += dpp_xchg<0x141>(s);
+                s += dpp_xchg<0x140>(s);
+                s = valid ? s * scale : kNoScore;
+                sc[j] = s;
+                grow |= s > m[j];
+            }
+            if (__any(grow)) { // some row's maximum moves: rescale what was summed so far
+#pragma unroll
+                for (int j = 0; j < QG; j++) {
+                    const float m_new = fmaxf(m[j], sc[j]);
+                    const float c = exp2_fast(m[j] - m_new);
+                    l[j] *= c;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[j][e] *= c;
+                    m[j] = m_new;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < QG; j++) {
+                const float p = valid ? exp2_fast(sc[j] - m[j]) : 0.f;
+                l[j] += p;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[j][e] = fmaf(p, v[e], acc[j][e]);
+            }
+        }
+    }
+
+    // merge the 4 rows of the wave (lanes 16 and 32 apart hold the same dims)
+#pragma unroll
+    for (int step = 16; step <= 32; step *= 2) {
+#pragma unroll
+        for (int j = 0; j < QG; j++) {
+            const float mo = __shfl_xor(m[j], step);
+            const float lo = __shfl_xor(l[j], step);
+            const float M = fmaxf(m[j], mo);
+            const float w1 = exp2_fast(m[j] - M), w2 = exp2_fast(mo - M);
+            l[j] = l[j] * w1 + lo * w2;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float ao = __shfl_xor(acc[j][e], step);
+                acc[j][e] = acc[j][e] * w1 + ao * w2;
+            }
+            m[j] = M;
+        }
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < QG; j++) {
+            *reinterpret_cast<float4 *>(&comb[wave][j][ds * 8]) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+            *reinterpret_cast<float4 *>(&comb[wave][j][ds * 8 + 4]) =
+                make_float4(acc[j][4], acc[j][5], acc[j][6], acc[j][7]);
+            if (ds == 0) {
+                comb[wave][j][HS] = m[j];
+                comb[wave][j][HS + 1] = l[j];
+            }
+        }
+    }
+    __syncthreads();
+    // merge the 4 waves; one thread per (head, dim)
+    for (int idx = tid; idx < QG * HS; idx += 256) {
+        const int j = idx >> 7, d = idx & 127;
+        float M = comb[0][j][HS];
+#pragma unroll
+        for (int w = 1; w < 4; w++) M = fmaxf(M, comb[w][j][HS]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float e = exp2_fast(comb[w][j][HS] - M);
+            num = fmaf(e, comb[w][j][d], num);
+            den = fmaf(e, comb[w][j][HS + 1], den);
+        }
+        const int h = kvh * QG + j;
+        if (A.n_splits == 1) {
+            const int i = h * HS + d;
+            A.out[A.scatter ? A.scatter[i] : i] = num / den;
+        } else {
+            float *p = A.part + ((size_t)h * A.max_splits + sp) * (HS + 2);
+            p[d] = num;
+            if (d == 0) {
+                p[HS] = M;
+                p[HS + 1] = den;
+            }
+        }
+    }
+}
+
+// Merge the splits of one q head: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s.
+// Wave 0 turns the (m_s, l_s) of up to 64 splits into weights; 4 groups of 128
+// threads then sum the weighted partial outputs, every load independent.
+__global__ __launch_bounds__(512) void attn_combine_kernel(const AttnDecode A) {
+    constexpr int HS = 128;
+    __shared__ float w[64];
+    __shared__ float den_s;
+    __shared__ float red[3][HS];
+    const int h = blockIdx.x, tid = threadIdx.x, d = tid & 127, grp = tid >> 7;
+    const int pos = A.dpos[0];
+    const int ns = min(A.n_splits, pos / A.ts + 1);
+    const float *p = A.part + (size_t)h * A.max_splits * (HS + 2);
+    if (tid < 64) {
+        const bool on = tid < ns;
+        const float ms = on ? p[tid * (HS + 2) + HS] : kNoScore;
+        const float ls = on ? p[tid * (HS + 2) + HS + 1] : 0.f;
+        const float M = wave_max(ms);
+        const float ws = on ? exp2_fast(ms - M) : 0.f;
+        w[tid] = ws;
+        const float den = wave_sum(ws * ls);
+        if (tid == 0) den_s = den;
+    }
+    __syncthreads();
+    float num = 0.f;
+#pragma unroll 4
+    for (int s = grp; s < ns; s += 4) num = fmaf(w[s], p[s * (HS + 2) + d], num);
+    if (grp > 0) red[grp - 1][d] = num;
+    __syncthreads();
+    if (grp == 0) {
+        num += red[0][d];
+        num += red[1][d];
+        num += red[2][d];
+        const int i = h * HS + d;
+        A.out[A.scatter ? A.scatter[i] : i] = num / den_s;
+    }
+}
+
+} // namespace
+
+int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
+    const int qg = a.n_heads / a.n_kv_heads;
+    if (a.ts < 64 || a.ts % 64 || a.n_splits < 1 || a.n_splits > a.max_splits || a.max_splits > 64)
+        return l2_fail(L2_ERR_ARG, "attention: ts=%d splits=%d/%d", a.ts, a.n_splits, a.max_splits);
+    dim3 grid(a.n_kv_heads, a.n_splits), block(256);
+    switch (qg) {
+        case 1: hipLaunchKernelGGL(attn_decode_kernel<1>, grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL(attn_decode_kernel<2>, grid, block, 0, st, a); break;
+        case 4: hipLaunchKernelGGL(attn_decode_kernel<4>, grid, block, 0, st, a); break;
+        case 8: hipLaunchKernelGGL(attn_decode_kernel<8>, grid, block, 0, st, a); break;
+        default: return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
+    }
+    L2_HIP(hipGetLastError());
+    if (a.n_splits > 1) {
+        hipLaunchKernelGGL(attn_combine_kernel, dim3(a.n_heads), dim3(512), 0, st, a);
+        L2_HIP(hipGetLastError());
+    }
+    return L2_OK;
+}

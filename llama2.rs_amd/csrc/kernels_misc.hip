@@ -196,191 +196,6 @@ __global__ __launch_bounds__(256) void attention_kernel(float *out, const float 
     }
 }
 
-// ---------------------------------------------------------------------------
-// Decode attention: one query position, all q heads of one kv head per block,
-// the timesteps cut into splits across grid.y (src/models.rs:131-176 computed
-// as softmax over partial maxima, which is the same function).
-//
-// RoPE (src/models.rs:100-129) is applied to q as it is staged, and to the new
-// key on its way into the cache (:236-249); the block that owns t == pos is the
-// only writer of that cache row and uses the fresh values directly.
-
-template <int QG>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
-    constexpr int HS = 128, HALF = 64;
-    extern __shared__ float sc[]; // [QG][ts] scores -> exp(score - max)
-    __shared__ float qs[QG * HS];
-    __shared__ float knew[HS];
-    __shared__ float ml[QG][2];
-    __shared__ float vred[7][HS];
-    const int kvh = blockIdx.x, sp = blockIdx.y;
-    const int pos = A.dpos[0];
-    const int t0 = sp * A.ts;
-    if (t0 > pos) return;
-    const int t1 = min(t0 + A.ts, pos + 1);
-    const int n = t1 - t0;
-    const int kv_dim = A.n_kv_heads * HS;
-    const int tid = threadIdx.x;
-    const float *ct = A.cos_t + (size_t)pos * HALF;
-    const float *st = A.sin_t + (size_t)pos * HALF;
-    for (int idx = tid; idx < QG * HALF; idx += 256) {
-        const int j = idx >> 6, i = idx & 63;
-        const float *qh = A.q + (size_t)(kvh * QG + j) * HS;
-        const float c = ct[i], s = st[i];
-        const float a = qh[i], b = qh[i + HALF];
-        const float first = a * c - b * s;
-        qs[j * HS + i] = first;
-        qs[j * HS + HALF + i] = b * c + first * s; // the in-place quirk: rotated first half
-    }
-    const bool owns_new = (t1 == pos + 1);
-    if (owns_new) {
-        if (tid < HALF) {
-            const float *kh = A.k_new + (size_t)kvh * HS;
-            const float c = ct[tid], s = st[tid];
-            const float a = kh[tid], b = kh[tid + HALF];
-            const float first = a * c - b * s;
-            const float second = b * c + first * s;
-            knew[tid] = first;
-            knew[tid + HALF] = second;
-            float *kc = A.kcache + (size_t)pos * kv_dim + kvh * HS;
-            kc[tid] = first;
-            kc[tid + HALF] = second;
-        } else if (tid >= 128) {
-            const int d = tid - 128;
-            A.vcache[(size_t)pos * kv_dim + kvh * HS + d] = A.v_new[(size_t)kvh * HS + d];
-        }
-    }
-    __syncthreads();
-
-    // scores: 4 lanes per timestep, 32 dims each, all QG heads against one load of K
-    const int sub = tid & 3;
-    const float root = sqrtf((float)HS);
-    for (int tt = tid >> 2; tt < n; tt += 64) {
-        const int t = t0 + tt;
-        float4 kk[8];
-        if (t == pos) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) kk[i] = reinterpret_cast<const float4 *>(knew + sub * 32)[i];
-        } else {
-            const float4 *kr = reinterpret_cast<const float4 *>(A.kcache + (size_t)t * kv_dim + kvh * HS + sub * 32);
-#pragma unroll
-            for (int i = 0; i < 8; i++) kk[i] = kr[i];
-        }
-#pragma unroll
-        for (int j = 0; j < QG; j++) {
-            const float4 *qr = reinterpret_cast<const float4 *>(qs + j * HS + sub * 32);
-            float s = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float4 qq = qr[i];
-                s = fmaf(qq.x, kk[i].x, s);
-                s = fmaf(qq.y, kk[i].y, s);
-                s = fmaf(qq.z, kk[i].z, s);
-                s = fmaf(qq.w, kk[i].w, s);
-            }
-            s += dpp_xchg<0xB1>(s);
-            s += dpp_xchg<0x4E>(s);
-            if (sub == 0) sc[j * A.ts + tt] = s / root;
-        }
-    }
-    __syncthreads();
-
-    // per head: max, exp, sum (wave w takes heads w, w+4)
-    const int lane = tid & 63, wave = tid >> 6;
-    for (int j = wave; j < QG; j += 4) {
-        float *row = sc + j * A.ts;
-        float m = -INFINITY;
-        for (int tt = lane; tt < n; tt += 64) m = fmaxf(m, row[tt]);
-        m = wave_max(m);
-        float l = 0.f;
-        for (int tt = lane; tt < n; tt += 64) {
-            const float e = expf(row[tt] - m);
-            row[tt] = e;
-            l += e;
-        }
-        l = wave_sum(l);
-        if (lane == 0) {
-            ml[j][0] = m;
-            ml[j][1] = l;
-        }
-    }
-    __syncthreads();
-
-    // weighted values: thread -> (4 dims, one of 8 interleaved sets of timesteps)
-    const int d4 = tid & 31, tg = tid >> 5;
-    float4 acc[QG];
-#pragma unroll
-    for (int j = 0; j < QG; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float *vbase = A.vcache + (size_t)kvh * HS + d4 * 4;
-#pragma unroll 2
-    for (int tt = tg; tt < n; tt += 8) {
-        const int t = t0 + tt;
-        const float4 v = (t == pos) ? *reinterpret_cast<const float4 *>(A.v_new + (size_t)kvh * HS + d4 * 4)
-                                    : *reinterpret_cast<const float4 *>(vbase + (size_t)t * kv_dim);
-#pragma unroll
-        for (int j = 0; j < QG; j++) {
-            const float p = sc[j * A.ts + tt];
-            acc[j].x = fmaf(p, v.x, acc[j].x);
-            acc[j].y = fmaf(p, v.y, acc[j].y);
-            acc[j].z = fmaf(p, v.z, acc[j].z);
-            acc[j].w = fmaf(p, v.w, acc[j].w);
-        }
-    }
-    // fold the 8 sets: sets 1..7 park their sums, set 0 adds them in order
-#pragma unroll
-    for (int j = 0; j < QG; j++) {
-        __syncthreads();
-        if (tg > 0) *reinterpret_cast<float4 *>(&vred[tg - 1][d4 * 4]) = acc[j];
-        __syncthreads();
-        if (tg == 0) {
-            float4 o = acc[j];
-#pragma unroll
-            for (int k = 0; k < 7; k++) {
-                const float4 e = *reinterpret_cast<const float4 *>(&vred[k][d4 * 4]);
-                o.x += e.x;
-                o.y += e.y;
-                o.z += e.z;
-                o.w += e.w;
-            }
-            const int h = kvh * QG + j;
-            const float vals[4] = {o.x, o.y, o.z, o.w};
-            if (A.n_splits == 1) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int i = h * HS + d4 * 4 + e;
-                    A.out[A.scatter ? A.scatter[i] : i] = vals[e] / ml[j][1];
-                }
-            } else {
-                float *p = A.part + ((size_t)h * A.max_splits + sp) * (HS + 2);
-                *reinterpret_cast<float4 *>(p + d4 * 4) = o;
-                if (d4 == 0) {
-                    p[HS] = ml[j][0];
-                    p[HS + 1] = ml[j][1];
-                }
-            }
-        }
-    }
-}
-
-// Merge the splits of one q head: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s.
-__global__ __launch_bounds__(128) void attn_combine_kernel(const AttnDecode A) {
-    constexpr int HS = 128;
-    const int h = blockIdx.x, d = threadIdx.x;
-    const int pos = A.dpos[0];
-    const int ns = min(A.n_splits, pos / A.ts + 1);
-    const float *p = A.part + (size_t)h * A.max_splits * (HS + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < ns; s++) M = fmaxf(M, p[s * (HS + 2) + HS]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < ns; s++) {
-        const float w = expf(p[s * (HS + 2) + HS] - M);
-        num = fmaf(w, p[s * (HS + 2) + d], num);
-        den = fmaf(w, p[s * (HS + 2) + HS + 1], den);
-    }
-    const int i = h * HS + d;
-    A.out[A.scatter ? A.scatter[i] : i] = num / den;
-}
-
 // Order-preserving key for (value, index): larger value wins, equal values ->
 // larger index wins, which is util::argmax's last-index rule (src/util.rs:39-46).
 __device__ __forceinline__ unsigned long long amax_key(float v, int idx) {
@@ -538,28 +353,6 @@ int attention_launch(float *out, const float *q, const float *kcache_l, const fl
     hipLaunchKernelGGL(attention_kernel, dim3(n_heads, B), dim3(256), lds, st, out, q, kcache_l, vcache_l,
                        pos, scatter, n_heads, n_kv_heads);
     L2_HIP(hipGetLastError());
-    return L2_OK;
-}
-
-int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
-    const int qg = a.n_heads / a.n_kv_heads;
-    if (a.ts < 64 || a.ts % 64 || a.n_splits < 1 || a.n_splits > a.max_splits)
-        return l2_fail(L2_ERR_ARG, "attention: ts=%d splits=%d/%d", a.ts, a.n_splits, a.max_splits);
-    const size_t lds = (size_t)qg * a.ts * sizeof(float);
-    if (lds > 40 * 1024) return l2_fail(L2_ERR_ARG, "attention: %d heads x %d timesteps per block", qg, a.ts);
-    dim3 grid(a.n_kv_heads, a.n_splits), block(256);
-    switch (qg) {
-        case 1: hipLaunchKernelGGL(attn_decode_kernel<1>, grid, block, lds, st, a); break;
-        case 2: hipLaunchKernelGGL(attn_decode_kernel<2>, grid, block, lds, st, a); break;
-        case 4: hipLaunchKernelGGL(attn_decode_kernel<4>, grid, block, lds, st, a); break;
-        case 8: hipLaunchKernelGGL(attn_decode_kernel<8>, grid, block, lds, st, a); break;
-        default: return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
-    }
-    L2_HIP(hipGetLastError());
-    if (a.n_splits > 1) {
-        hipLaunchKernelGGL(attn_combine_kernel, dim3(a.n_heads), dim3(128), 0, st, a);
-        L2_HIP(hipGetLastError());
-    }
     return L2_OK;
 }
 

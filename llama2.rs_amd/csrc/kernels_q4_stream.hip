@@ -205,18 +205,25 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         }
     };
 
-    // prime the pipe before anything else: these loads do not depend on x
+    // x first, then the first rows of the weights: loads return in order, and
+    // the staging of x (a cache hit) must not queue behind rows that come from HBM.
+    StageRegs xr[NM];
+#pragma unroll
+    for (int q = 0; q < NM; q++) stage_issue<NW>(L.m[mi + q].x + (size_t)b * in, L.m[mi + q].wn, in, 0, tid, xr[q]);
+    __builtin_amdgcn_sched_barrier(0);
     RowData pipe[P][NM];
 #pragma unroll
     for (int u = 0; u < P; u++) fetch(u, pipe[u]);
+    __builtin_amdgcn_sched_barrier(0);
 
     // stage x for the whole block, then take this lane's chunk into registers
     float ssq = 0.f;
 #pragma unroll
     for (int q = 0; q < NM; q++) {
         const Q4Mat &M = L.m[mi + q];
-        const float p = stage_input<NW>(M.x + (size_t)b * in, M.wn, in, lds + q * xstride,
-                                        lds + q * xstride + C * kChunkPad, tid);
+        float *xs = lds + q * xstride;
+        float p = stage_consume<NW>(M.wn != nullptr, in, 0, tid, xr[q], xs, xs + C * kChunkPad, 0.f);
+        p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
         if (q == 0) ssq = p;
     }
     const bool norm = L.m[mi].wn != nullptr;

@@ -59,49 +59,83 @@ __device__ __forceinline__ float chunk_dot(const uint4 w, const float (&x)[32]) 
 
 // Stage one input vector into padded chunks + chunk sums; returns this
 // thread's share of sum(x^2) (of the raw input, before the norm weight).
+constexpr int kStageBatch = 4; // float4 loads of x (and of the norm weight) in flight per thread
+
+struct StageRegs {
+    float4 v[kStageBatch], g[kStageBatch];
+};
+
+// Issue the loads of batch `base` (in float4 units) into registers.
 template <int NW>
-__device__ __forceinline__ float stage_input(const float *__restrict__ xin_f, const float *__restrict__ wn_f,
-                                             int in, float *xs, float *xsum, int tid) {
+__device__ __forceinline__ void stage_issue(const float *__restrict__ xin_f, const float *__restrict__ wn_f,
+                                            int in, int base, int tid, StageRegs &r) {
     const float4 *xin = reinterpret_cast<const float4 *>(xin_f);
     const float4 *wn = reinterpret_cast<const float4 *>(wn_f);
     const int n4 = in >> 2;
-    constexpr int T = NW * 64, U = 4;
-    float ssq = 0.f;
-    for (int base = 0; base < n4; base += T * U) {
-        float4 v[U], g[U];
-        // all loads of a batch are issued before the first one is consumed
+    constexpr int T = NW * 64;
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int j4 = base + u * T + tid;
-            v[u] = j4 < n4 ? xin[j4] : make_float4(0.f, 0.f, 0.f, 0.f);
-            g[u] = (wn_f && j4 < n4) ? wn[j4] : make_float4(1.f, 1.f, 1.f, 1.f);
+    for (int u = 0; u < kStageBatch; u++) {
+        const int j4 = base + u * T + tid;
+        r.v[u] = j4 < n4 ? xin[j4] : make_float4(0.f, 0.f, 0.f, 0.f);
+        r.g[u] = (wn_f && j4 < n4) ? wn[j4] : make_float4(1.f, 1.f, 1.f, 1.f);
+    }
+}
+
+// Consume a batch: norm weight, sum of squares, chunk sums, LDS.
+template <int NW>
+__device__ __forceinline__ float stage_consume(bool norm, int in, int base, int tid, StageRegs &r, float *xs,
+                                               float *xsum, float ssq) {
+    const int n4 = in >> 2;
+    constexpr int T = NW * 64;
+#pragma unroll
+    for (int u = 0; u < kStageBatch; u++) {
+        const int j4 = base + u * T + tid;
+        float4 v = r.v[u];
+        if (norm) {
+            ssq = fmaf(v.x, v.x, ssq);
+            ssq = fmaf(v.y, v.y, ssq);
+            ssq = fmaf(v.z, v.z, ssq);
+            ssq = fmaf(v.w, v.w, ssq);
+            v.x *= r.g[u].x;
+            v.y *= r.g[u].y;
+            v.z *= r.g[u].z;
+            v.w *= r.g[u].w;
         }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int j4 = base + u * T + tid;
-            if (wn_f) {
-                ssq = fmaf(v[u].x, v[u].x, ssq);
-                ssq = fmaf(v[u].y, v[u].y, ssq);
-                ssq = fmaf(v[u].z, v[u].z, ssq);
-                ssq = fmaf(v[u].w, v[u].w, ssq);
-                v[u].x *= g[u].x;
-                v[u].y *= g[u].y;
-                v[u].z *= g[u].z;
-                v[u].w *= g[u].w;
-            }
-            // the 8 consecutive lanes that hold one chunk add up its sum
-            float s = (v[u].x + v[u].y) + (v[u].z + v[u].w);
-            s += dpp_xchg<0xB1>(s);  // lanes ^1
-            s += dpp_xchg<0x4E>(s);  // lanes ^2
-            s += dpp_xchg<0x141>(s); // 7 - lane within each 8: the other quad
-            if (j4 < n4) {
-                const int j = j4 << 2;
-                *reinterpret_cast<float4 *>(&xs[(j >> 5) * kChunkPad + (j & 31)]) = v[u];
-                if ((tid & 7) == 0) xsum[j >> 5] = s;
-            }
+        // the 8 consecutive lanes that hold one chunk add up its sum
+        float s = (v.x + v.y) + (v.z + v.w);
+        s += dpp_xchg<0xB1>(s);  // lanes ^1
+        s += dpp_xchg<0x4E>(s);  // lanes ^2
+        s += dpp_xchg<0x141>(s); // 7 - lane within each 8: the other quad
+        if (j4 < n4) {
+            const int j = j4 << 2;
+            *reinterpret_cast<float4 *>(&xs[(j >> 5) * kChunkPad + (j & 31)]) = v;
+            if ((tid & 7) == 0) xsum[j >> 5] = s;
         }
     }
     return ssq;
+}
+
+// Whatever the first batch did not cover.
+template <int NW>
+__device__ __forceinline__ float stage_rest(const float *__restrict__ xin_f, const float *__restrict__ wn_f, int in,
+                                            float *xs, float *xsum, int tid, float ssq) {
+    const int n4 = in >> 2;
+    constexpr int T = NW * 64;
+    for (int base = T * kStageBatch; base < n4; base += T * kStageBatch) {
+        StageRegs r;
+        stage_issue<NW>(xin_f, wn_f, in, base, tid, r);
+        ssq = stage_consume<NW>(wn_f != nullptr, in, base, tid, r, xs, xsum, ssq);
+    }
+    return ssq;
+}
+
+template <int NW>
+__device__ __forceinline__ float stage_input(const float *__restrict__ xin_f, const float *__restrict__ wn_f,
+                                             int in, float *xs, float *xsum, int tid) {
+    StageRegs r;
+    stage_issue<NW>(xin_f, wn_f, in, 0, tid, r);
+    const float ssq = stage_consume<NW>(wn_f != nullptr, in, 0, tid, r, xs, xsum, 0.f);
+    return stage_rest<NW>(xin_f, wn_f, in, xs, xsum, tid, ssq);
 }
 
 } // namespace q4
