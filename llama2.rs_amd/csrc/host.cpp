@@ -945,7 +945,7 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
             a.q = m->qv, a.k_new = m->kv, a.v_new = m->vv;
             a.kcache = kc, a.vcache = vc;
             a.cos_t = m->rope_cos, a.sin_t = m->rope_sin;
-            a.dpos = m->dpos;
+            a.pos = max_pos;
             a.out = m->attg, a.scatter = wo.inv_index;
             a.part = m->attn_part;
             a.n_heads = d.n_heads, a.n_kv_heads = d.n_kv_heads;

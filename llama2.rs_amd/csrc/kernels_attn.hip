@@ -52,20 +52,23 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// Layout of a block: 4 waves x 4 rows of 16 lanes.  One row of lanes handles
+// Layout of a block: NWV waves x 4 rows of 16 lanes.  One row of lanes handles
 // one timestep at a time, each lane 8 of the 128 head dimensions; a block
-// covers 16 timesteps per step and PD steps per tile, all of a tile's loads
-// being issued before its arithmetic.  All QG query heads of the kv head share
+// covers 4 NWV timesteps per step and PD steps per tile, all of a tile's loads
+// being issued before its arithmetic.  NWV is 4 when the timesteps are cut
+// into splits; wider blocks were measured slower for the single block per kv
+// head of a short context (more waves to start and to merge).  All QG query heads of the kv head share
 // each K and V load (grouped-query attention, src/models.rs:142-145).
-template <int QG>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
+template <int QG, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode A) {
+    constexpr int NT = NWV * 64, TSTEP = NWV * 4;
     constexpr int HS = 128, HALF = 64;
-    constexpr int PD = QG >= 8 ? 2 : 4;
+    constexpr int PD = QG >= 8 ? 2 : 4; // steps in flight (8 was measured slower at short contexts: coarser tiles)
     __shared__ float qs[QG * HS];
     __shared__ float kvnew[2][HS];
-    __shared__ float comb[4][QG][HS + 2];
+    __shared__ float comb[NWV][QG][HS + 2];
     const int kvh = blockIdx.x, sp = blockIdx.y;
-    const int pos = A.dpos[0];
+    const int pos = A.pos;
     const int t0 = sp * A.ts;
     if (t0 > pos) return;
     const int t1 = min(t0 + A.ts, pos + 1);
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     const int kv_dim = A.n_kv_heads * HS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ds = lane & 15;            // dims [8 ds, 8 ds + 8)
-    const int tl = wave * 4 + (lane >> 4); // this row's timestep within a step of 16
+    const int tl = wave * 4 + (lane >> 4); // this row's timestep within a step
 
     const float *__restrict__ kc = A.kcache;
     const float *__restrict__ vc = A.vcache;
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     // Unconditional loads: rows past the end re-read the last row, and the row
     // of the new position is read although its values are replaced below.
     auto fetch = [&](int it, Step &d) {
-        const int t = min(t0 + it * 16 + tl, t_last);
+        const int t = min(t0 + it * TSTEP + tl, t_last);
         const uint32_t off = __umul24(t, row_bytes) + lane_off;
         d.k0 = ld_at<float4>(kc, off);
         d.k1 = ld_at<float4>(kc, off + 16);
@@ -100,11 +103,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     // thread's element), so that no load can move into a branch further down.
     const float *ct = A.cos_t + (size_t)pos * HALF;
     const float *st = A.sin_t + (size_t)pos * HALF;
-    constexpr int NQ = (QG * HALF + 255) / 256;
+    constexpr int NQ = (QG * HALF + NT - 1) / NT;
     float qa[NQ], qb[NQ], qc[NQ], qsn[NQ];
 #pragma unroll
     for (int r = 0; r < NQ; r++) {
-        const int idx = (tid + r * 256) % (QG * HALF);
+        const int idx = (tid + r * NT) % (QG * HALF);
         const int j = idx >> 6, i = idx & 63;
         const float *qh = A.q + (size_t)(kvh * QG + j) * HS;
         qa[r] = qh[i], qb[r] = qh[i + HALF];
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     // q with RoPE, src/models.rs:100-129 (the second half uses the rotated first half)
 #pragma unroll
     for (int r = 0; r < NQ; r++) {
-        const int idx = (tid + r * 256) % (QG * HALF);
+        const int idx = (tid + r * NT) % (QG * HALF);
         const int j = idx >> 6, i = idx & 63;
         const float first = qa[r] * qc[r] - qb[r] * qsn[r];
         qs[j * HS + i] = first;
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
                 float *kw = A.kcache + (size_t)pos * kv_dim + kvh * HS;
                 kw[tid] = first;
                 kw[tid + HALF] = second;
-            } else if (tid >= 128) {
+            } else if (tid >= 128 && tid < 256) {
                 A.vcache[(size_t)pos * kv_dim + kvh * HS + (tid - 128)] = nv;
             }
         }
@@ -173,7 +176,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
     }
     // log2(e) / sqrt(head_size): src/models.rs:154 divides the score by sqrt(head_size)
     const float scale = 1.44269504088896340736f / sqrtf((float)HS);
-    const int n_it = (n + 15) >> 4;
+    const int n_it = (n + TSTEP - 1) / TSTEP;
     const int n_tiles = (n_it + PD - 1) / PD;
     for (int tile = 0; tile < n_tiles; tile++) {
         if (tile > 0) { // all of the tile's loads, then its arithmetic
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
         }
 #pragma unroll
         for (int u = 0; u < PD; u++) {
-            const int t = t0 + (tile * PD + u) * 16 + tl;
+            const int t = t0 + (tile * PD + u) * TSTEP + tl;
             const bool valid = t < t1;
             const Step &d = pipe[u];
             float k[8] = {d.k0.x, d.k0.y, d.k0.z, d.k0.w, d.k1.x, d.k1.y, d.k1.z, d.k1.w};
@@ -274,15 +277,15 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnDecode A) {
         }
     }
     __syncthreads();
-    // merge the 4 waves; one thread per (head, dim)
-    for (int idx = tid; idx < QG * HS; idx += 256) {
+    // merge the waves; one thread per (head, dim)
+    for (int idx = tid; idx < QG * HS; idx += NT) {
         const int j = idx >> 7, d = idx & 127;
         float M = comb[0][j][HS];
 #pragma unroll
-        for (int w = 1; w < 4; w++) M = fmaxf(M, comb[w][j][HS]);
+        for (int w = 1; w < NWV; w++) M = fmaxf(M, comb[w][j][HS]);
         float num = 0.f, den = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
+        for (int w = 0; w < NWV; w++) {
             const float e = exp2_fast(comb[w][j][HS] - M);
             num = fmaf(e, comb[w][j][d], num);
             den = fmaf(e, comb[w][j][HS + 1], den);
@@ -311,7 +314,7 @@ __global__ __launch_bounds__(512) void attn_combine_kernel(const AttnDecode A) {
     __shared__ float den_s;
     __shared__ float red[3][HS];
     const int h = blockIdx.x, tid = threadIdx.x, d = tid & 127, grp = tid >> 7;
-    const int pos = A.dpos[0];
+    const int pos = A.pos;
     const int ns = min(A.n_splits, pos / A.ts + 1);
     const float *p = A.part + (size_t)h * A.max_splits * (HS + 2);
     if (tid < 64) {
@@ -339,21 +342,26 @@ __global__ __launch_bounds__(512) void attn_combine_kernel(const AttnDecode A) {
     }
 }
 
+template <int QG>
+int attn_launch_qg(const AttnDecode &a, hipStream_t st) {
+    hipLaunchKernelGGL((attn_decode_kernel<QG, 4>), dim3(a.n_kv_heads, a.n_splits), dim3(256), 0, st, a);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
 } // namespace
 
 int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
     const int qg = a.n_heads / a.n_kv_heads;
     if (a.ts < 64 || a.ts % 64 || a.n_splits < 1 || a.n_splits > a.max_splits || a.max_splits > 64)
         return l2_fail(L2_ERR_ARG, "attention: ts=%d splits=%d/%d", a.ts, a.n_splits, a.max_splits);
-    dim3 grid(a.n_kv_heads, a.n_splits), block(256);
     switch (qg) {
-        case 1: hipLaunchKernelGGL(attn_decode_kernel<1>, grid, block, 0, st, a); break;
-        case 2: hipLaunchKernelGGL(attn_decode_kernel<2>, grid, block, 0, st, a); break;
-        case 4: hipLaunchKernelGGL(attn_decode_kernel<4>, grid, block, 0, st, a); break;
-        case 8: hipLaunchKernelGGL(attn_decode_kernel<8>, grid, block, 0, st, a); break;
+        case 1: L2_TRY(attn_launch_qg<1>(a, st)); break;
+        case 2: L2_TRY(attn_launch_qg<2>(a, st)); break;
+        case 4: L2_TRY(attn_launch_qg<4>(a, st)); break;
+        case 8: L2_TRY(attn_launch_qg<8>(a, st)); break;
         default: return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
     }
-    L2_HIP(hipGetLastError());
     if (a.n_splits > 1) {
         hipLaunchKernelGGL(attn_combine_kernel, dim3(a.n_heads), dim3(512), 0, st, a);
         L2_HIP(hipGetLastError());

@@ -131,6 +131,16 @@ __device__ __forceinline__ void st_at(float *base, uint32_t byte_offset, float v
     *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + byte_offset) = v;
 }
 
+#if defined(Q4S_TS) // measurement build only: per-block timestamps (100 MHz counter)
+__device__ unsigned long long q4s_ts[1024 * 8];
+#define Q4S_STAMP(k)                                                                  \
+    do {                                                                              \
+        if (threadIdx.x == 0 && blockIdx.x < 1024) q4s_ts[blockIdx.x * 8 + (k)] = wall_clock64(); \
+    } while (0)
+#else
+#define Q4S_STAMP(k)
+#endif
+
 struct RowData {
     uint4 w;
     float s;
@@ -152,6 +162,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     __shared__ float red[NW];
     __shared__ float part[2][TR][NM][PW];
 
+    Q4S_STAMP(0);
     const int in = L.in;
     const int C = in >> 5;
     const int xstride = C * kChunkPad + C;
@@ -226,6 +237,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
         if (q == 0) ssq = p;
     }
+    Q4S_STAMP(1);
     const bool norm = L.m[mi].wn != nullptr;
     if (norm) {
         ssq = wave_sum(ssq);
@@ -298,7 +310,9 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     // was staged). The compiler's wait counts inside the loop are then those of
     // the steady state alone: vmcnt leaves the P - 1 younger rows in flight.
     // Otherwise the issue order of the prologue leaks into the loop's waits.
+    Q4S_STAMP(2);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0), expcnt and lgkmcnt untouched
+    Q4S_STAMP(3);
     // Epilogue operands, uniform for the block.
     const Q4Epi &E = L.e;
     const int epi_kind = E.kind;
@@ -389,8 +403,17 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
                 if (t < n_scatter) st_at(sc_out[t], ((uint32_t)out_base + sidx[t]) << 2, v); // 32-bit offset: nothing widens the loaded index
         }
         buf ^= 1;
+        Q4S_STAMP(4 + (tile + 1 == n_tiles));
     }
 }
+
+#if defined(Q4S_TS)
+} // namespace
+extern "C" int l2_debug_q4_ts(unsigned long long *out, int n) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(q4s_ts), (size_t)n * 8);
+}
+namespace {
+#endif
 
 int cu_count() {
     static int n = 0;

@@ -142,7 +142,7 @@ struct AttnDecode {
     const float *v_new;  // [kv_dim] value
     float *kcache, *vcache;          // this layer: [max_seq][kv_dim]
     const float *cos_t, *sin_t;      // [max_seq][head_size/2]
-    const int32_t *dpos;             // device: position of this step
+    int pos;                         // position of this step (the host knows it; no device read in front of the loads)
     float *out;                      // [dim], written through scatter
     const int32_t *scatter;
     float *part;                     // split workspace: [n_heads][max_splits][130]

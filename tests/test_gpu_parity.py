@@ -135,6 +135,39 @@ def test_forward_logits_and_cache_vs_oracle(ops, oracle, dims, tmp_path):
     o.close()
 
 
+@pytest.mark.parametrize("n_heads,n_kv,ctx", [(2, 2, 300), (8, 2, 257), (8, 1, 1000), (4, 2, 4300)],
+                         ids=["mha_5splits", "gqa4_first_split", "gqa8_16splits", "gqa2_deep"])
+def test_decode_attention_long_context(ops, oracle, n_heads, n_kv, ctx):
+    """Decode steps behind a long cache: the timesteps are cut across blocks and merged.  The cache rows
+    are synthetic (written on the device, copied into the oracle's cache), so no long prompt is needed."""
+    dims = ck.Dims(dim=128 * n_heads, hidden_dim=512, n_layers=2, n_heads=n_heads, n_kv_heads=n_kv,
+                   vocab_size=300, seq_len=ctx + 8, group_size=128)
+    img = ck.synth_weights_image(dims, seed=7)
+    m = ops.Model(img, dims)
+    o = oracle.Model(img, dims)
+    o.new_state()
+    m.fill_kv_synthetic(0, ctx, seed=3)
+    ko, vo = o.kv_cache()
+    for l in range(dims.n_layers):
+        k, v = m.read_kv(l, 0, ctx)
+        ko[l, :ctx] = k
+        vo[l, :ctx] = v
+    tok = 11
+    for pos in range(ctx, ctx + 3):
+        want = o.transformer([tok], [pos])
+        got = m.forward([tok], [pos])
+        assert nrel(got, want) < REL_FP32, pos
+        tok = oracle.argmax(want)
+        assert int(np.argmax(got)) == tok
+    # the rows written behind the synthetic ones
+    for l in range(dims.n_layers):
+        k, v = m.read_kv(l, ctx, 3)
+        assert nrel(k, ko[l, ctx:ctx + 3]) < REL_FP32
+        assert nrel(v, vo[l, ctx:ctx + 3]) < REL_FP32
+    m.close()
+    o.close()
+
+
 def test_model_operator_entry_points(ops, oracle):
     dims = TINY_GQA
     img = ck.synth_weights_image(dims, seed=3)
