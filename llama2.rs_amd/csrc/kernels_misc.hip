@@ -206,77 +206,72 @@ __device__ __forceinline__ unsigned long long amax_key(float v, int idx) {
 }
 
 // Linear::matvec (src/model.rs:22-31) for the classifier: one wave per row,
-// two rows in flight, x staged in LDS.  With wn set, x is first normalised as
-// rmsnorm does (src/models.rs:53-66, :288-295): the block stages wn[i]*x[i] and
-// scales each logit by ss = 1/sqrt(mean(x^2) + eps).  Optionally folds each
-// logit into a 64-bit (value,index) maximum.
+// x staged in LDS.  With wn set, x is first normalised as rmsnorm does
+// (src/models.rs:53-66, :288-295): the block stages wn[i]*x[i] and scales each
+// logit by ss = 1/sqrt(mean(x^2) + eps).  Optionally folds each logit into a
+// 64-bit (value,index) maximum, one atomic per wave.
+//
+// A wave takes R rows at a time and issues all R * KI loads of 16 bytes per
+// lane (32 in all) before the first FMA, every load unconditional: columns past
+// the end re-read the row's last 16 bytes against a zero of x, rows past the
+// end re-read the last row.
+template <int KI> // float4 per lane and row
 __global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float *w, const float *x,
                                                             const float *wn, float eps, int in, int out,
                                                             unsigned long long *amax) {
-    extern __shared__ float xs[];
+    constexpr int R = 32 / KI >= 1 ? 32 / KI : 1;
+    extern __shared__ float xs[]; // KI * 64 float4, zero beyond in
     __shared__ float red[16];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    float ssq = 0.f;
-    for (int i = tid; i < in / 4; i += 256) {
-        float4 v = reinterpret_cast<const float4 *>(x)[i];
-        if (wn) {
-            const float4 g = reinterpret_cast<const float4 *>(wn)[i];
-            ssq = fmaf(v.x, v.x, ssq);
-            ssq = fmaf(v.y, v.y, ssq);
-            ssq = fmaf(v.z, v.z, ssq);
-            ssq = fmaf(v.w, v.w, ssq);
-            v.x *= g.x;
-            v.y *= g.y;
-            v.z *= g.z;
-            v.w *= g.w;
-        }
-        reinterpret_cast<float4 *>(xs)[i] = v;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: row addresses stay scalar
+    const int n4 = in >> 2;
+    const float4 *__restrict__ w4 = reinterpret_cast<const float4 *>(w);
+    const float4 *__restrict__ xs4 = reinterpret_cast<const float4 *>(xs);
+
+    constexpr int XL = (KI * 64 + 255) / 256;
+    float4 xv[XL], gv[XL];
+#pragma unroll
+    for (int r = 0; r < XL; r++) {
+        const int i = min(tid + r * 256, n4 - 1);
+        xv[r] = reinterpret_cast<const float4 *>(x)[i];
+        gv[r] = wn ? reinterpret_cast<const float4 *>(wn)[i] : make_float4(1.f, 1.f, 1.f, 1.f);
     }
-    float ss = 1.0f;
-    if (wn) {
-        ssq = block_sum(ssq, red);
-        ssq /= (float)in;
-        ssq += eps;
-        ss = 1.0f / sqrtf(ssq);
-    }
-    __syncthreads();
-    const int n4 = in / 4;
+
     const int waves_total = gridDim.x * 4;
-    constexpr int RW = 4; // rows per wave and pass: RW x 2 loads of 16 bytes in flight per lane
-    for (int o = (blockIdx.x * 4 + wave) * RW; o < out; o += waves_total * RW) {
-        const float4 *r[RW];
-        float a[RW];
+    const int o_first = (blockIdx.x * 4 + wave) * R;
+    uint32_t col[KI]; // byte offsets within a row
 #pragma unroll
-        for (int k = 0; k < RW; k++) {
-            r[k] = reinterpret_cast<const float4 *>(w + (size_t)min(o + k, out - 1) * in);
-            a[k] = 0.f;
+    for (int i = 0; i < KI; i++) col[i] = (uint32_t)min(i * 64 + lane, n4 - 1) << 4;
+    float4 wv[R][KI];
+    auto load_tile = [&](int o) {
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+            // 32-bit byte offsets from the one base (the launcher checks that the matrix stays below 4 GiB)
+            const uint32_t row = (uint32_t)min(o + k, out - 1) * ((uint32_t)n4 << 4);
+#pragma unroll
+            for (int i = 0; i < KI; i++)
+                wv[k][i] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(w4) + (row + col[i]));
         }
-        for (int j = lane; j < n4; j += 128) {
-            const int j2 = j + 64;
-            const bool two = j2 < n4;
-            float4 wv[RW][2];
+    };
+    float ss = 1.0f;
+    unsigned long long key = 0ull;
+    auto finish_tile = [&](int o) {
+        float a[R];
 #pragma unroll
-            for (int k = 0; k < RW; k++) {
-                wv[k][0] = r[k][j];
-                wv[k][1] = two ? r[k][j2] : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-            const float4 x0 = reinterpret_cast<const float4 *>(xs)[j];
-            const float4 x1 = two ? reinterpret_cast<const float4 *>(xs)[j2] : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int k = 0; k < R; k++) a[k] = 0.f;
 #pragma unroll
-            for (int k = 0; k < RW; k++) {
-                a[k] = fmaf(wv[k][0].x, x0.x, a[k]);
-                a[k] = fmaf(wv[k][0].y, x0.y, a[k]);
-                a[k] = fmaf(wv[k][0].z, x0.z, a[k]);
-                a[k] = fmaf(wv[k][0].w, x0.w, a[k]);
-                a[k] = fmaf(wv[k][1].x, x1.x, a[k]);
-                a[k] = fmaf(wv[k][1].y, x1.y, a[k]);
-                a[k] = fmaf(wv[k][1].z, x1.z, a[k]);
-                a[k] = fmaf(wv[k][1].w, x1.w, a[k]);
+        for (int i = 0; i < KI; i++) {
+            const float4 xx = xs4[i * 64 + lane];
+#pragma unroll
+            for (int k = 0; k < R; k++) {
+                a[k] = fmaf(wv[k][i].x, xx.x, a[k]);
+                a[k] = fmaf(wv[k][i].y, xx.y, a[k]);
+                a[k] = fmaf(wv[k][i].z, xx.z, a[k]);
+                a[k] = fmaf(wv[k][i].w, xx.w, a[k]);
             }
         }
-        unsigned long long key = 0ull;
 #pragma unroll
-        for (int k = 0; k < RW; k++) {
+        for (int k = 0; k < R; k++) {
             const float v = wave_sum(a[k]) * ss;
             if (lane == 0 && o + k < out) {
                 y[o + k] = v;
@@ -284,8 +279,39 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float
                 key = kk > key ? kk : key;
             }
         }
-        if (lane == 0 && amax) atomicMax(amax, key);
+    };
+    float ssq = 0.f;
+#pragma unroll
+    for (int r = 0; r < XL; r++) {
+        const int i = tid + r * 256;
+        float4 v = xv[r];
+        if (i >= n4) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (wn) {
+            ssq = fmaf(v.x, v.x, ssq);
+            ssq = fmaf(v.y, v.y, ssq);
+            ssq = fmaf(v.z, v.z, ssq);
+            ssq = fmaf(v.w, v.w, ssq);
+            v.x *= gv[r].x;
+            v.y *= gv[r].y;
+            v.z *= gv[r].z;
+            v.w *= gv[r].w;
+        }
+        if (i < KI * 64) reinterpret_cast<float4 *>(xs)[i] = v;
     }
+    if (wn) {
+        ssq = block_sum(ssq, red);
+        ssq /= (float)in;
+        ssq += eps;
+        ss = 1.0f / sqrtf(ssq);
+    }
+    __syncthreads();
+    for (int o = o_first; o < out; o += waves_total * R) {
+        __builtin_amdgcn_sched_barrier(0); // a tile's loads stay behind the tile before it: one set of registers
+        load_tile(o);
+        __builtin_amdgcn_sched_barrier(0); // every load of the tile before its first FMA
+        finish_tile(o);
+    }
+    if (lane == 0 && amax && key) atomicMax(amax, key);
 }
 
 // Greedy hand-over (src/inference.rs:154-162, 185-189): next is the forced
@@ -358,11 +384,24 @@ int attention_launch(float *out, const float *q, const float *kcache_l, const fl
 
 int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
                         unsigned long long *amax_key, hipStream_t st) {
-    if (in % 4 || in * 4 > 64 * 1024) return l2_fail(L2_ERR_ARG, "dense matvec: in=%d", in);
-    int blocks = (out + 15) / 16;
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(dense_matvec_kernel, dim3(blocks), dim3(256), (size_t)in * 4, st, y, w, x, wn, eps, in,
-                       out, amax_key);
+    if (in < 4 || in % 4 || in > 8192 || out < 1 || (size_t)in * out * 4 >= ((size_t)1 << 32))
+        return l2_fail(L2_ERR_ARG, "dense matvec: in=%d out=%d", in, out);
+    const int ki = (in / 4 + 63) / 64; // float4 per lane and row
+    const int KI = ki <= 4 ? 4 : ki <= 8 ? 8 : ki <= 16 ? 16 : ki <= 20 ? 20 : 32;
+    const int R = 32 / KI >= 1 ? 32 / KI : 1;
+    // three blocks per CU (the registers allow three waves per SIMD), fewer when the rows run out
+    int blocks = 3 * 256;
+    const int need = (out + 4 * R - 1) / (4 * R);
+    if (blocks > need) blocks = need;
+    const size_t lds = (size_t)KI * 64 * 16;
+    dim3 grid(blocks), block(256);
+    switch (KI) {
+        case 4: hipLaunchKernelGGL(dense_matvec_kernel<4>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
+        case 8: hipLaunchKernelGGL(dense_matvec_kernel<8>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
+        case 16: hipLaunchKernelGGL(dense_matvec_kernel<16>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
+        case 20: hipLaunchKernelGGL(dense_matvec_kernel<20>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
+        default: hipLaunchKernelGGL(dense_matvec_kernel<32>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
+    }
     L2_HIP(hipGetLastError());
     return L2_OK;
 }
