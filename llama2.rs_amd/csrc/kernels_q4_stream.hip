@@ -147,8 +147,14 @@ struct RowData {
     int32_t z;
 };
 
-template <int G, int NWK, int S, bool PAIR, bool IDOT>
+// MODE 0: fp32 inner loop, x staged through LDS (rmsnorm prologue, several matrices, row pairs).
+// MODE 1: integer-dot inner loop, x staged and quantised in LDS.
+// MODE 2: fp32 inner loop, one matrix without rmsnorm: every lane loads its own 32 values of x
+//         straight into registers; no LDS staging, no barrier before the first row.
+template <int G, int NWK, int S, bool PAIR, int MODE>
 __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L) {
+    constexpr bool IDOT = MODE == 1, DIRECT = MODE == 2;
+    static_assert(!(DIRECT && PAIR), "the direct form takes one matrix");
     constexpr int NM = PAIR ? 2 : 1;
     constexpr int NW = NWK * S;
 #ifndef Q4S_P
@@ -218,87 +224,113 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
 
     // x first, then the first rows of the weights: loads return in order, and
     // the staging of x (a cache hit) must not queue behind rows that come from HBM.
-    StageRegs xr[NM];
+    StageRegs xr[DIRECT ? 1 : NM];
+    float4 xd[DIRECT ? 8 : 1];
+    if constexpr (DIRECT) {
+        const float4 *xp = reinterpret_cast<const float4 *>(L.m[mi].x + (size_t)b * in) + cc * 8;
 #pragma unroll
-    for (int q = 0; q < NM; q++) stage_issue<NW>(L.m[mi + q].x + (size_t)b * in, L.m[mi + q].wn, in, 0, tid, xr[q]);
+        for (int i = 0; i < 8; i++) xd[i] = xp[i];
+    } else {
+#pragma unroll
+        for (int q = 0; q < NM; q++)
+            stage_issue<NW>(L.m[mi + q].x + (size_t)b * in, L.m[mi + q].wn, in, 0, tid, xr[q]);
+    }
     __builtin_amdgcn_sched_barrier(0);
+    Q4S_STAMP(6);
     RowData pipe[P][NM];
 #pragma unroll
     for (int u = 0; u < P; u++) fetch(u, pipe[u]);
     __builtin_amdgcn_sched_barrier(0);
+    Q4S_STAMP(7);
 
-    // stage x for the whole block, then take this lane's chunk into registers
-    float ssq = 0.f;
-#pragma unroll
-    for (int q = 0; q < NM; q++) {
-        const Q4Mat &M = L.m[mi + q];
-        float *xs = lds + q * xstride;
-        float p = stage_consume<NW>(M.wn != nullptr, in, 0, tid, xr[q], xs, xs + C * kChunkPad, 0.f);
-        p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
-        if (q == 0) ssq = p;
-    }
-    Q4S_STAMP(1);
-    const bool norm = L.m[mi].wn != nullptr;
-    if (norm) {
-        ssq = wave_sum(ssq);
-        if (lane == 0) red[wave] = ssq;
-    }
-    __syncthreads();
-    float ss = 1.0f;
-    if (norm) { // rmsnorm scale, src/models.rs:55-60
-        float t = 0.f;
-#pragma unroll
-        for (int i = 0; i < NW; i++) t += red[i];
-        t /= (float)in;
-        t += L.eps;
-        ss = 1.0f / sqrtf(t);
-    }
     // this lane's slice of x, for good: 32 floats, or 24 digit words + step + sum of q
     float x[NM][IDOT ? 1 : 32];
     int xp[NM][IDOT ? 24 : 1];
     float sx[NM];     // fp32 form: sum of the chunk's x; integer form: sum of its q
     float xdelta[NM]; // integer form: the chunk's step
-    if constexpr (IDOT) {
+    float ss = 1.0f;
+    const bool norm = !DIRECT && L.m[mi].wn != nullptr;
+    if constexpr (DIRECT) {
+        float t = 0.f;
 #pragma unroll
-        for (int q = 0; q < NM; q++) quantize_in_place<NW * 64>(lds + q * xstride, C, tid);
-    }
+        for (int i = 0; i < 8; i++) {
+            const float4 v = has_chunk ? xd[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            x[0][4 * i + 0] = v.x;
+            x[0][4 * i + 1] = v.y;
+            x[0][4 * i + 2] = v.z;
+            x[0][4 * i + 3] = v.w;
+            t += (v.x + v.y) + (v.z + v.w);
+        }
+        sx[0] = t;
+        xdelta[0] = 0.f;
+        Q4S_STAMP(1);
+    } else {
+        // stage x for the whole block, then take this lane's chunk into registers
+        float ssq = 0.f;
 #pragma unroll
-    for (int q = 0; q < NM; q++) {
-        const float *xs = lds + q * xstride;
-        xdelta[q] = 0.f;
-        sx[q] = 0.f;
+        for (int q = 0; q < NM; q++) {
+            const Q4Mat &M = L.m[mi + q];
+            float *xs = lds + q * xstride;
+            float p = stage_consume<NW>(M.wn != nullptr, in, 0, tid, xr[q], xs, xs + C * kChunkPad, 0.f);
+            p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
+            if (q == 0) ssq = p;
+        }
+        Q4S_STAMP(1);
+        if (norm) {
+            ssq = wave_sum(ssq);
+            if (lane == 0) red[wave] = ssq;
+        }
+        __syncthreads();
+        if (norm) { // rmsnorm scale, src/models.rs:55-60
+            float t = 0.f;
+#pragma unroll
+            for (int i = 0; i < NW; i++) t += red[i];
+            t /= (float)in;
+            t += L.eps;
+            ss = 1.0f / sqrtf(t);
+        }
         if constexpr (IDOT) {
-            if (has_chunk) {
-                const uint4 *p = reinterpret_cast<const uint4 *>(&xs[c * kPlaneWords]);
 #pragma unroll
-                for (int i = 0; i < 6; i++) {
-                    const uint4 v = p[i];
-                    xp[q][4 * i + 0] = (int)v.x;
-                    xp[q][4 * i + 1] = (int)v.y;
-                    xp[q][4 * i + 2] = (int)v.z;
-                    xp[q][4 * i + 3] = (int)v.w;
+            for (int q = 0; q < NM; q++) quantize_in_place<NW * 64>(lds + q * xstride, C, tid);
+        }
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            const float *xs = lds + q * xstride;
+            xdelta[q] = 0.f;
+            sx[q] = 0.f;
+            if constexpr (IDOT) {
+                if (has_chunk) {
+                    const uint4 *p = reinterpret_cast<const uint4 *>(&xs[c * kPlaneWords]);
+#pragma unroll
+                    for (int i = 0; i < 6; i++) {
+                        const uint4 v = p[i];
+                        xp[q][4 * i + 0] = (int)v.x;
+                        xp[q][4 * i + 1] = (int)v.y;
+                        xp[q][4 * i + 2] = (int)v.z;
+                        xp[q][4 * i + 3] = (int)v.w;
+                    }
+                    xdelta[q] = xs[c * kPlaneWords + 24];
+                    sx[q] = xs[c * kPlaneWords + 25];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 24; i++) xp[q][i] = 0;
                 }
-                xdelta[q] = xs[c * kPlaneWords + 24];
-                sx[q] = xs[c * kPlaneWords + 25];
             } else {
+                if (has_chunk) {
+                    const float4 *p = reinterpret_cast<const float4 *>(&xs[c * kChunkPad]);
 #pragma unroll
-                for (int i = 0; i < 24; i++) xp[q][i] = 0;
-            }
-        } else {
-            if (has_chunk) {
-                const float4 *p = reinterpret_cast<const float4 *>(&xs[c * kChunkPad]);
+                    for (int i = 0; i < 8; i++) {
+                        const float4 v = p[i];
+                        x[q][4 * i + 0] = v.x;
+                        x[q][4 * i + 1] = v.y;
+                        x[q][4 * i + 2] = v.z;
+                        x[q][4 * i + 3] = v.w;
+                    }
+                    sx[q] = xs[C * kChunkPad + c];
+                } else {
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const float4 v = p[i];
-                    x[q][4 * i + 0] = v.x;
-                    x[q][4 * i + 1] = v.y;
-                    x[q][4 * i + 2] = v.z;
-                    x[q][4 * i + 3] = v.w;
+                    for (int i = 0; i < 32; i++) x[q][i] = 0.f;
                 }
-                sx[q] = xs[C * kChunkPad + c];
-            } else {
-#pragma unroll
-                for (int i = 0; i < 32; i++) x[q][i] = 0.f;
             }
         }
     }
@@ -427,12 +459,12 @@ int cu_count() {
     return n;
 }
 
-template <int G, int NWK, int S, bool PAIR, bool IDOT>
+template <int G, int NWK, int S, bool PAIR, int MODE>
 int launch_s(Q4Launch &L, hipStream_t stream) {
     constexpr int NW = NWK * S;
     constexpr int TR = (PAIR ? Q4S_P / 2 : Q4S_P) * S;
     const int C = L.in / 32;
-    const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
+    const size_t lds = MODE == 2 ? 0 : (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
     if (lds + 8 * 1024 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
     // Blocks: a whole number of rounds over the CUs, as many blocks per CU as
     // 16 waves and the LDS allow; every block gets the same number of rows.
@@ -454,7 +486,7 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     }
     L.rows_per_block = rpb;
     for (int i = 0; i < L.n_mats; i++) L.m[i].row_blocks = (L.m[i].out + rpb - 1) / rpb;
-    auto kern = q4_stream_kernel<G, NWK, S, PAIR, IDOT>;
+    auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE>;
     if (lds > 48 * 1024) {
         static size_t raised = 0; // per instantiation
         if (lds > raised) {
@@ -474,26 +506,28 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     return L2_OK;
 }
 
-template <int G, bool IDOT>
+template <int G, int MODE>
 int launch_sg(Q4Launch &L, hipStream_t stream) {
     const int nwk = (L.in / 32 + 63) / 64;
-    if (!L.pair) {
+    if constexpr (MODE == 2) {
+        if (!L.pair && nwk >= 9 && nwk <= 14) return launch_s<G, 14, 1, false, MODE>(L, stream);
+    } else if (!L.pair) {
         switch (nwk) {
-            case 1: return launch_s<G, 1, 4, false, IDOT>(L, stream);
-            case 2: return launch_s<G, 2, 4, false, IDOT>(L, stream);
-            case 3: return launch_s<G, 3, 4, false, IDOT>(L, stream);
-            case 4: return launch_s<G, 4, 4, false, IDOT>(L, stream);
-            case 5: case 6: return launch_s<G, 6, 2, false, IDOT>(L, stream);
-            case 7: return launch_s<G, 7, 2, false, IDOT>(L, stream);
-            case 8: return launch_s<G, 8, 2, false, IDOT>(L, stream);
-            case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, IDOT>(L, stream);
+            case 1: return launch_s<G, 1, 4, false, MODE>(L, stream);
+            case 2: return launch_s<G, 2, 4, false, MODE>(L, stream);
+            case 3: return launch_s<G, 3, 4, false, MODE>(L, stream);
+            case 4: return launch_s<G, 4, 4, false, MODE>(L, stream);
+            case 5: case 6: return launch_s<G, 6, 2, false, MODE>(L, stream);
+            case 7: return launch_s<G, 7, 2, false, MODE>(L, stream);
+            case 8: return launch_s<G, 8, 2, false, MODE>(L, stream);
+            case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, MODE>(L, stream);
         }
     } else {
         switch (nwk) {
-            case 1: return launch_s<G, 1, 4, true, IDOT>(L, stream);
-            case 2: return launch_s<G, 2, 4, true, IDOT>(L, stream);
-            case 3: return launch_s<G, 3, 2, true, IDOT>(L, stream);
-            case 4: return launch_s<G, 4, 2, true, IDOT>(L, stream);
+            case 1: return launch_s<G, 1, 4, true, MODE>(L, stream);
+            case 2: return launch_s<G, 2, 4, true, MODE>(L, stream);
+            case 3: return launch_s<G, 3, 2, true, MODE>(L, stream);
+            case 4: return launch_s<G, 4, 2, true, MODE>(L, stream);
         }
     }
     return l2_fail(L2_ERR_ARG, "q4 matvec (streaming): in=%d pair=%d has no kernel", L.in, L.pair);
@@ -507,17 +541,27 @@ int q4_stream_launch(Q4Launch &L, hipStream_t stream) {
         const char *v = getenv("L2_Q4_IMPL");
         return !(v && !strcmp(v, "idot"));
     }();
-    if (fp32_form) {
+    // One matrix, no rmsnorm in front, and an input so long that its staging (over 64 KB of LDS per block)
+    // costs more than lanes fetching their own 128 bytes: x goes straight to registers.  For shorter inputs
+    // the strided 16-byte loads of that form were measured slower than the LDS staging (4096: 7.5 vs 5.9 us).
+    const bool direct = fp32_form && !L.pair && L.n_mats == 1 && L.m[0].wn == nullptr && L.in > 16384;
+    if (direct) {
         switch (L.group_size) {
-            case 32: return launch_sg<32, false>(L, stream);
-            case 64: return launch_sg<64, false>(L, stream);
-            case 128: return launch_sg<128, false>(L, stream);
+            case 32: return launch_sg<32, 2>(L, stream);
+            case 64: return launch_sg<64, 2>(L, stream);
+            case 128: return launch_sg<128, 2>(L, stream);
+        }
+    } else if (fp32_form) {
+        switch (L.group_size) {
+            case 32: return launch_sg<32, 0>(L, stream);
+            case 64: return launch_sg<64, 0>(L, stream);
+            case 128: return launch_sg<128, 0>(L, stream);
         }
     } else {
         switch (L.group_size) {
-            case 32: return launch_sg<32, true>(L, stream);
-            case 64: return launch_sg<64, true>(L, stream);
-            case 128: return launch_sg<128, true>(L, stream);
+            case 32: return launch_sg<32, 1>(L, stream);
+            case 64: return launch_sg<64, 1>(L, stream);
+            case 128: return launch_sg<128, 1>(L, stream);
         }
     }
     return l2_fail(L2_ERR_ARG, "q4 matvec: group size %d (32, 64 or 128)", L.group_size);
