@@ -151,16 +151,13 @@ struct RowData {
 // MODE 1: integer-dot inner loop, x staged and quantised in LDS.
 // MODE 2: fp32 inner loop, one matrix without rmsnorm: every lane loads its own 32 values of x
 //         straight into registers; no LDS staging, no barrier before the first row.
-template <int G, int NWK, int S, bool PAIR, int MODE>
+template <int G, int NWK, int S, bool PAIR, int MODE, int P>
 __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L) {
     constexpr bool IDOT = MODE == 1, DIRECT = MODE == 2;
     static_assert(!(DIRECT && PAIR), "the direct form takes one matrix");
     constexpr int NM = PAIR ? 2 : 1;
     constexpr int NW = NWK * S;
-#ifndef Q4S_P
-#define Q4S_P 4
-#endif
-    constexpr int P = PAIR ? Q4S_P / 2 : Q4S_P; // rows (row pairs) in flight per stream
+    // P rows (row pairs) are in flight per stream
     constexpr int TR = P * S;       // rows per reduction tile
     constexpr int PW = NWK * 4;     // partials per row
     constexpr int CPG = G / 32;     // chunks per group
@@ -459,34 +456,57 @@ int cu_count() {
     return n;
 }
 
-template <int G, int NWK, int S, bool PAIR, int MODE>
-int launch_s(Q4Launch &L, hipStream_t stream) {
-    constexpr int NW = NWK * S;
-    constexpr int TR = (PAIR ? Q4S_P / 2 : Q4S_P) * S;
-    const int C = L.in / 32;
-    const size_t lds = MODE == 2 ? 0 : (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
-    if (lds + 8 * 1024 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
-    // Blocks: a whole number of rounds over the CUs, as many blocks per CU as
-    // 16 waves and the LDS allow; every block gets the same number of rows.
+// Rows per block for a block of NW waves and tiles of TR rows: a whole number of rounds over the CUs, as
+// many blocks per CU as 16 waves and the LDS allow; every block gets the same number of rows; several
+// matrices round up separately and the grid stays within one round.
+static int plan_rows(const Q4Launch &L, int NW, int TR, size_t lds, bool pair, int *total_out) {
     int per_cu = 16 / NW;
     if (per_cu < 1) per_cu = 1;
     const int by_lds = (int)((150 * 1024) / (lds + 4 * 1024));
     if (per_cu > by_lds) per_cu = by_lds < 1 ? 1 : by_lds;
     long rows = 0;
-    for (int i = 0; i < (PAIR ? 1 : L.n_mats); i++) rows += L.m[i].out;
+    const int nm = pair ? 1 : L.n_mats;
+    for (int i = 0; i < nm; i++) rows += L.m[i].out;
     const long slots = (long)cu_count() * per_cu;
     int rpb = (int)((rows + slots - 1) / slots);
     if (rpb < TR) rpb = TR;
     int total = 0;
-    for (;;) { // several matrices round up separately: keep the grid within one round
+    for (;;) {
         total = 0;
-        for (int i = 0; i < (PAIR ? 1 : L.n_mats); i++) total += (L.m[i].out + rpb - 1) / rpb;
+        for (int i = 0; i < nm; i++) total += (L.m[i].out + rpb - 1) / rpb;
         if (total <= slots || rpb >= rows) break;
         rpb++;
     }
+    if (total_out) *total_out = total;
+    return rpb;
+}
+
+// Wave-rows of arithmetic per CU for a candidate shape: what the choice between shapes minimises.
+static long plan_cost(const Q4Launch &L, int NWK, int S, int P, bool pair) {
+    const int C = L.in / 32;
+    const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float) * (pair ? 2 : 1);
+    const int NW = NWK * S, TR = P * S;
+    int per_cu = 16 / NW;
+    if (per_cu < 1) per_cu = 1;
+    const int by_lds = (int)((150 * 1024) / (lds + 4 * 1024));
+    if (per_cu > by_lds) per_cu = by_lds < 1 ? 1 : by_lds;
+    const int rpb = plan_rows(L, NW, TR, lds, pair, nullptr);
+    const long tiles = (rpb + TR - 1) / TR;
+    return (long)per_cu * NW * tiles * P;
+}
+
+template <int G, int NWK, int S, bool PAIR, int MODE, int P = (PAIR ? 2 : 4)>
+int launch_s(Q4Launch &L, hipStream_t stream) {
+    constexpr int NW = NWK * S;
+    constexpr int TR = P * S;
+    const int C = L.in / 32;
+    const size_t lds = MODE == 2 ? 0 : (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
+    if (lds + 8 * 1024 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
+    int total = 0;
+    const int rpb = plan_rows(L, NW, TR, lds, PAIR, &total);
     L.rows_per_block = rpb;
     for (int i = 0; i < L.n_mats; i++) L.m[i].row_blocks = (L.m[i].out + rpb - 1) / rpb;
-    auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE>;
+    auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE, P>;
     if (lds > 48 * 1024) {
         static size_t raised = 0; // per instantiation
         if (lds > raised) {
@@ -515,10 +535,12 @@ int launch_sg(Q4Launch &L, hipStream_t stream) {
         switch (nwk) {
             case 1: return launch_s<G, 1, 4, false, MODE>(L, stream);
             case 2: return launch_s<G, 2, 4, false, MODE>(L, stream);
-            case 3: return launch_s<G, 3, 4, false, MODE>(L, stream);
+            case 3: // 5120: 20 rows per block are one tile of 5 streams, 60 or so are four tiles either way
+                if (plan_cost(L, 3, 5, 4, false) < plan_cost(L, 3, 4, 4, false)) return launch_s<G, 3, 5, false, MODE>(L, stream);
+                return launch_s<G, 3, 4, false, MODE>(L, stream);
             case 4: return launch_s<G, 4, 4, false, MODE>(L, stream);
             case 5: case 6: return launch_s<G, 6, 2, false, MODE>(L, stream);
-            case 7: return launch_s<G, 7, 2, false, MODE>(L, stream);
+            case 7: return launch_s<G, 7, 2, false, MODE, 5>(L, stream); // 13824 -> 5120: 20 rows per block in two tiles
             case 8: return launch_s<G, 8, 2, false, MODE>(L, stream);
             case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, MODE>(L, stream);
         }
@@ -526,7 +548,7 @@ int launch_sg(Q4Launch &L, hipStream_t stream) {
         switch (nwk) {
             case 1: return launch_s<G, 1, 4, true, MODE>(L, stream);
             case 2: return launch_s<G, 2, 4, true, MODE>(L, stream);
-            case 3: return launch_s<G, 3, 2, true, MODE>(L, stream);
+            case 3: return launch_s<G, 3, 5, true, MODE>(L, stream);
             case 4: return launch_s<G, 4, 2, true, MODE>(L, stream);
         }
     }
