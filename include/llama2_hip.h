@@ -133,6 +133,11 @@ int l2_state_reset(l2_state *s);
  * [npos][n_kv_heads][head_size].  For tests (the reference's fields are
  * private, src/models.rs:29-33). */
 int l2_state_read_kv(l2_state *s, int layer, int pos0, int npos, float *k_host, float *v_host);
+/* The inverse: overwrite cache rows [pos0, pos0+npos) of one layer from host
+ * arrays of the same shape.  With l2_state_read_kv this snapshots and restores
+ * a RunState (the reference clones the boxed struct, src/models.rs:29-42), so
+ * that a shared prompt prefix is computed once. */
+int l2_state_write_kv(l2_state *s, int layer, int pos0, int npos, const float *k_host, const float *v_host);
 /* Overwrite cache rows [pos0, pos0+npos) of every layer with a deterministic
  * pattern in (-1, 1) derived from seed: stands in for a long prompt when a
  * benchmark needs a deep cache without paying for its prefill. */

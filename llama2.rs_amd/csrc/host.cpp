@@ -714,6 +714,19 @@ extern "C" int l2_state_read_kv(l2_state *s, int layer, int pos0, int npos, floa
     return L2_OK;
 }
 
+extern "C" int l2_state_write_kv(l2_state *s, int layer, int pos0, int npos, const float *k_host,
+                                 const float *v_host) {
+    if (!s || !k_host || !v_host) return l2_fail(L2_ERR_ARG, "null argument");
+    const l2_model *m = s->m;
+    if (layer < 0 || layer >= m->d.n_layers || pos0 < 0 || npos < 0 || pos0 + npos > m->max_seq)
+        return l2_fail(L2_ERR_RANGE, "write_kv: layer %d, positions [%d,%d)", layer, pos0, pos0 + npos);
+    const size_t off = ((size_t)layer * m->max_seq + pos0) * m->kv_dim;
+    L2_HIP(hipStreamSynchronize(m->stream));
+    L2_HIP(hipMemcpy(s->kcache + off, k_host, (size_t)npos * m->kv_dim * 4, hipMemcpyHostToDevice));
+    L2_HIP(hipMemcpy(s->vcache + off, v_host, (size_t)npos * m->kv_dim * 4, hipMemcpyHostToDevice));
+    return L2_OK;
+}
+
 extern "C" int l2_state_fill_synthetic(l2_state *s, int pos0, int npos, uint64_t seed) {
     if (!s) return l2_fail(L2_ERR_ARG, "null state");
     const l2_model *m = s->m;

@@ -591,5 +591,8 @@ int q4_stream_launch(Q4Launch &L, hipStream_t stream) {
 
 bool q4_stream_supports(const Q4Launch &L) {
     const int nwk = (L.in / 32 + 63) / 64;
+    // the kernel addresses a matrix with 32-bit byte offsets and 24-bit row numbers
+    for (int i = 0; i < L.n_mats; i++)
+        if (L.m[i].out >= (1 << 24) || (size_t)L.m[i].out * (size_t)(L.in / 8) * 4 >= ((size_t)1 << 32)) return false;
     return L.pair ? nwk <= 4 : nwk <= 14;
 }

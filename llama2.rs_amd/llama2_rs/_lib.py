@@ -60,6 +60,7 @@ SIGNATURES = {
     "l2_state_free": (None, [_VP]),
     "l2_state_reset": (_I, [_VP]),
     "l2_state_read_kv": (_I, [_VP, _I, _I, _I, _VP, _VP]),
+    "l2_state_write_kv": (_I, [_VP, _I, _I, _I, _VP, _VP]),
     "l2_state_fill_synthetic": (_I, [_VP, _I, _I, C.c_uint64]),
     "l2_qlinear_create": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, C.POINTER(_VP)]),
     "l2_qlinear_free": (None, [_VP]),

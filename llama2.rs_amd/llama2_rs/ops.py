@@ -209,6 +209,14 @@ class Model:
         check(lib().l2_state_read_kv(self.state, layer, pos0, npos, _p(k), _p(v)))
         return k, v
 
+    def write_kv(self, layer: int, pos0: int, k, v):
+        d = self.dims
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        if k.shape != v.shape or k.shape[1:] != (d.n_kv_heads, d.head_size):
+            raise ValueError(f"k, v must be [npos][{d.n_kv_heads}][{d.head_size}]")
+        check(lib().l2_state_write_kv(self.state, layer, pos0, k.shape[0], _p(k), _p(v)))
+
     def fill_kv_synthetic(self, pos0: int, npos: int, seed: int = 0):
         check(lib().l2_state_fill_synthetic(self.state, pos0, npos, seed))
 

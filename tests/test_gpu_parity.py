@@ -168,6 +168,35 @@ def test_decode_attention_long_context(ops, oracle, n_heads, n_kv, ctx):
     o.close()
 
 
+def test_kv_snapshot_restore(ops):
+    """read_kv / write_kv: a cache restored into a fresh state continues with the same tokens."""
+    dims = TINY_GQA
+    img = ck.synth_weights_image(dims, seed=9)
+    m = ops.Model(img, dims)
+    prompt = np.array([4, 9, 200, 31, 7, 7, 100], np.int32)
+    full, _ = m.generate_greedy(prompt, 24, use_prefill=False)
+    # replay the first 12 positions, snapshot, restore into another model's state, continue from there
+    m.reset()
+    tok = 1
+    for pos in range(12):
+        nxt = m.decode_greedy(tok, pos)
+        tok = int(prompt[pos]) if pos < len(prompt) else nxt
+    snap = [m.read_kv(l, 0, 12) for l in range(dims.n_layers)]
+    m2 = ops.Model(img, dims)
+    for l, (k, v) in enumerate(snap):
+        m2.write_kv(l, 0, k, v)
+    out = []
+    for pos in range(12, 24):
+        tok = m2.decode_greedy(tok, pos)
+        out.append(tok)
+    np.testing.assert_array_equal(out, full[12:24])
+    from llama2_rs._lib import L2Error
+    with pytest.raises(L2Error):
+        m2.write_kv(0, dims.seq_len - 1, snap[0][0][:2], snap[0][1][:2])
+    m.close()
+    m2.close()
+
+
 def test_model_operator_entry_points(ops, oracle):
     dims = TINY_GQA
     img = ck.synth_weights_image(dims, seed=3)
