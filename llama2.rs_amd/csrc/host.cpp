@@ -982,7 +982,7 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
         } else {
             LAUNCH(K_ROPE_KV, rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
                                              d.n_kv_heads, m->head_size, B, st));
-            LAUNCH(K_ATTENTION, attention_launch(m->attg, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads,
+            LAUNCH(K_ATTENTION, attention_launch(m->attg, nullptr, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads,
                                                  d.n_kv_heads, m->head_size, max_pos, B, st));
         }
         {   // wo (:260) + residual (:263-264); the new x also goes out in w1's and w3's order
@@ -1078,9 +1078,14 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
                          &w3 = m->q[L2_W3][l];
         const float *wn = m->dwn + (size_t)l * 5 * dim;
         L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
-        L2_TRY(prep_f16_launch(m->h16a, m->xq, wn + 0 * (size_t)dim, dim, B, st));
-        L2_TRY(prep_f16_launch(m->h16b, m->xk, wn + 1 * (size_t)dim, dim, B, st));
-        L2_TRY(prep_f16_launch(m->h16c, m->xv, wn + 2 * (size_t)dim, dim, B, st));
+        {
+            PrepList P{};
+            P.n_mats = 3;
+            P.out[0] = m->h16a, P.x[0] = m->xq, P.wn[0] = wn + 0 * (size_t)dim;
+            P.out[1] = m->h16b, P.x[1] = m->xk, P.wn[1] = wn + 1 * (size_t)dim;
+            P.out[2] = m->h16c, P.x[2] = m->xv, P.wn[2] = wn + 2 * (size_t)dim;
+            L2_TRY(prep_f16_multi_launch(P, dim, B, st));
+        }
         {
             Q4Launch Q = launch_of(wq, B, m->rms_eps);
             Q.m[0] = mat_of(wq, nullptr, nullptr, m->qv);
@@ -1094,9 +1099,8 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
         float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
         L2_TRY(rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
                               d.n_kv_heads, m->head_size, B, st));
-        L2_TRY(attention_launch(m->attg, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
+        L2_TRY(attention_launch(nullptr, m->h16a, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
                                 m->head_size, max_pos, B, st));
-        L2_TRY(prep_f16_launch(m->h16a, m->attg, nullptr, dim, B, st));
         {
             Q4Launch Q = launch_of(wo, B, 0.f);
             Q.m[0] = mat_of(wo, nullptr, nullptr, m->x);
@@ -1109,8 +1113,13 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
             L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
         }
         L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
-        L2_TRY(prep_f16_launch(m->h16a, m->x1, wn + 3 * (size_t)dim, dim, B, st));
-        L2_TRY(prep_f16_launch(m->h16b, m->x3, wn + 4 * (size_t)dim, dim, B, st));
+        {
+            PrepList P{};
+            P.n_mats = 2;
+            P.out[0] = m->h16a, P.x[0] = m->x1, P.wn[0] = wn + 3 * (size_t)dim;
+            P.out[1] = m->h16b, P.x[1] = m->x3, P.wn[1] = wn + 4 * (size_t)dim;
+            L2_TRY(prep_f16_multi_launch(P, dim, B, st));
+        }
         {
             Q4Launch Q = launch_of(w1, B, m->rms_eps);
             Q.m[0] = mat_of(w1, nullptr, nullptr, m->hb);
@@ -1119,8 +1128,7 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
             XhList X{{m->h16a, m->h16b, nullptr}};
             L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st));
         }
-        L2_TRY(silu_scatter_launch(m->hg, m->hb, m->hb2, w2.inv_index, hid, B, st));
-        L2_TRY(prep_f16_launch(m->h16a, m->hg, nullptr, hid, B, st));
+        L2_TRY(silu_scatter_launch(nullptr, m->h16a, m->hb, m->hb2, w2.inv_index, hid, B, st));
         {
             Q4Launch Q = launch_of(w2, B, 0.f);
             Q.m[0] = mat_of(w2, nullptr, nullptr, m->x);

@@ -305,6 +305,175 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
     }
 }
 
+// Attention for a chunk of B positions (prefill, src/models.rs:131-176 with B > 1).  Every cache row of
+// the chunk is already written and q already rotated (rope_kv_kernel).  The same layout as the decode
+// kernel, with the 8 "heads" of a block being 8 / QG query positions x the QG query heads of one kv head:
+// the K and V rows a block streams are shared by 8 score/value streams instead of being re-read per query.
+// Query j sees timesteps 0..pos[j] (causal within the chunk as well).
+template <int QG>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(float *__restrict__ out, _Float16 *__restrict__ out_h,
+                                                            const float *__restrict__ q,
+                                                            const float *__restrict__ kc, const float *__restrict__ vc,
+                                                            const int32_t *__restrict__ pos,
+                                                            const int32_t *__restrict__ scatter, int n_heads,
+                                                            int n_kv_heads, int B) {
+    constexpr int HS = 128, NQ = 8, QPB = NQ / QG, PD = 2, TSTEP = 16;
+    __shared__ float qs[NQ * HS];
+    __shared__ float comb[4][NQ][HS + 2];
+    __shared__ int pj_s[NQ];
+    const int kvh = blockIdx.x, qb = blockIdx.y;
+    const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ds = lane & 15;
+    const int tl = wave * 4 + (lane >> 4);
+    // stream j: query qb * QPB + j / QG, head kvh * QG + j % QG
+    if (tid < NQ) {
+        const int qi = qb * QPB + tid / QG;
+        pj_s[tid] = qi < B ? pos[qi] : -1;
+    }
+    for (int idx = tid; idx < NQ * HS; idx += 256) {
+        const int j = idx >> 7, d = idx & 127;
+        const int qi = min(qb * QPB + j / QG, B - 1);
+        qs[idx] = q[(size_t)qi * dim + (kvh * QG + j % QG) * HS + d];
+    }
+    __syncthreads();
+    int pj[NQ];
+    int t_end = 0; // one past the last timestep any stream of the block sees
+#pragma unroll
+    for (int j = 0; j < NQ; j++) {
+        pj[j] = pj_s[j];
+        t_end = max(t_end, pj[j] + 1);
+    }
+    if (t_end == 0) return;
+    const uint32_t row_bytes = (uint32_t)kv_dim * 4u;
+    const uint32_t lane_off = (uint32_t)(kvh * HS + ds * 8) * 4u;
+    struct Step {
+        float4 k0, k1, v0, v1;
+    };
+    auto fetch = [&](int it, Step &d) {
+        const int t = min(it * TSTEP + tl, t_end - 1);
+        const uint32_t off = __umul24(t, row_bytes) + lane_off;
+        d.k0 = ld_at<float4>(kc, off);
+        d.k1 = ld_at<float4>(kc, off + 16);
+        d.v0 = ld_at<float4>(vc, off);
+        d.v1 = ld_at<float4>(vc, off + 16);
+    };
+    float m[NQ], l[NQ], acc[NQ][8];
+#pragma unroll
+    for (int j = 0; j < NQ; j++) {
+        m[j] = kNoScore;
+        l[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[j][e] = 0.f;
+    }
+    const float scale = 1.44269504088896340736f / sqrtf((float)HS);
+    const int n_it = (t_end + TSTEP - 1) / TSTEP;
+    const int n_tiles = (n_it + PD - 1) / PD;
+    Step pipe[PD];
+    for (int tile = 0; tile < n_tiles; tile++) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PD; u++) fetch(tile * PD + u, pipe[u]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PD; u++) {
+            const int t = (tile * PD + u) * TSTEP + tl;
+            const Step &d = pipe[u];
+            const float k[8] = {d.k0.x, d.k0.y, d.k0.z, d.k0.w, d.k1.x, d.k1.y, d.k1.z, d.k1.w};
+            float v[8] = {d.v0.x, d.v0.y, d.v0.z, d.v0.w, d.v1.x, d.v1.y, d.v1.z, d.v1.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = t < t_end ? v[e] : 0.f; // rows past the end may hold anything
+            float sc[NQ];
+            bool grow = false;
+#pragma unroll
+            for (int j = 0; j < NQ; j++) {
+                const float4 a = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8]);
+                const float4 b = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8 + 4]);
+                const float qj[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) s = fmaf(qj[e], k[e], s);
+                s += dpp_xchg<0xB1>(s);
+                s += dpp_xchg<0x4E>(s);
+                s += dpp_xchg<0x141>(s);
+                s += dpp_xchg<0x140>(s);
+                s = t <= pj[j] ? s * scale : kNoScore;
+                sc[j] = s;
+                grow |= s > m[j];
+            }
+            if (__any(grow)) {
+#pragma unroll
+                for (int j = 0; j < NQ; j++) {
+                    const float m_new = fmaxf(m[j], sc[j]);
+                    const float c = exp2_fast(m[j] - m_new);
+                    l[j] *= c;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[j][e] *= c;
+                    m[j] = m_new;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NQ; j++) {
+                const float p = t <= pj[j] ? exp2_fast(sc[j] - m[j]) : 0.f;
+                l[j] += p;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[j][e] = fmaf(p, v[e], acc[j][e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int step = 16; step <= 32; step *= 2) {
+#pragma unroll
+        for (int j = 0; j < NQ; j++) {
+            const float mo = __shfl_xor(m[j], step);
+            const float lo = __shfl_xor(l[j], step);
+            const float M = fmaxf(m[j], mo);
+            const float w1 = exp2_fast(m[j] - M), w2 = exp2_fast(mo - M);
+            l[j] = l[j] * w1 + lo * w2;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float ao = __shfl_xor(acc[j][e], step);
+                acc[j][e] = acc[j][e] * w1 + ao * w2;
+            }
+            m[j] = M;
+        }
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < NQ; j++) {
+            *reinterpret_cast<float4 *>(&comb[wave][j][ds * 8]) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+            *reinterpret_cast<float4 *>(&comb[wave][j][ds * 8 + 4]) =
+                make_float4(acc[j][4], acc[j][5], acc[j][6], acc[j][7]);
+            if (ds == 0) {
+                comb[wave][j][HS] = m[j];
+                comb[wave][j][HS + 1] = l[j];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < NQ * HS; idx += 256) {
+        const int j = idx >> 7, d = idx & 127;
+        const int qi = qb * QPB + j / QG;
+        if (qi >= B) continue;
+        float M = comb[0][j][HS];
+#pragma unroll
+        for (int w = 1; w < 4; w++) M = fmaxf(M, comb[w][j][HS]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float e = exp2_fast(comb[w][j][HS] - M);
+            num = fmaf(e, comb[w][j][d], num);
+            den = fmaf(e, comb[w][j][HS + 1], den);
+        }
+        const int i = (kvh * QG + j % QG) * HS + d;
+        const int dst = scatter ? scatter[i] : i;
+        if (out_h) // straight into the fp16 pair-interleaved order the next GEMM reads
+            out_h[(size_t)qi * dim + h16_slot(dst)] = (_Float16)(num / den);
+        else
+            out[(size_t)qi * dim + dst] = num / den;
+    }
+}
+
 // Merge the splits of one q head: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s.
 // Wave 0 turns the (m_s, l_s) of up to 64 splits into weights; 4 groups of 128
 // threads then sum the weighted partial outputs, every load independent.
@@ -366,5 +535,25 @@ int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
         hipLaunchKernelGGL(attn_combine_kernel, dim3(a.n_heads), dim3(512), 0, st, a);
         L2_HIP(hipGetLastError());
     }
+    return L2_OK;
+}
+
+int attention_launch(float *out, void *out_f16, const float *q, const float *kcache_l, const float *vcache_l,
+                     const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
+                     int head_size, int max_pos, int B, hipStream_t st) {
+    (void)max_pos;
+    if (head_size != 128) return l2_fail(L2_ERR_ARG, "attention: head_size=%d (128 only)", head_size);
+    const int qg = n_heads / n_kv_heads;
+    if (qg != 1 && qg != 2 && qg != 4 && qg != 8)
+        return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
+    const int qpb = 8 / qg;
+    dim3 grid(n_kv_heads, (B + qpb - 1) / qpb), block(256);
+    switch (qg) {
+        case 1: hipLaunchKernelGGL(attn_prefill_kernel<1>, grid, block, 0, st, out, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B); break;
+        case 2: hipLaunchKernelGGL(attn_prefill_kernel<2>, grid, block, 0, st, out, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B); break;
+        case 4: hipLaunchKernelGGL(attn_prefill_kernel<4>, grid, block, 0, st, out, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B); break;
+        default: hipLaunchKernelGGL(attn_prefill_kernel<8>, grid, block, 0, st, out, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B); break;
+    }
+    L2_HIP(hipGetLastError());
     return L2_OK;
 }

@@ -1,6 +1,5 @@
 // The per-token kernels around the q4 matvec: embedding gather, RoPE + KV-cache
-// write, GQA attention (a split-KV decode kernel with RoPE folded in, and a
-// batched one for prefill chunks), the fp32 classifier with RMSNorm in front
+// write for prefill chunks, the fp32 classifier with RMSNorm in front
 // and the argmax behind, and the greedy loop's token hand-over.  gfx950, wave64.
 //
 // This file is compiled with -ffp-contract=off: wherever the reference rounds
@@ -127,74 +126,6 @@ __global__ void rope_kv_kernel(float *q, const float *k, const float *v, const i
     for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) vc[i] = vb[i];
 }
 
-// multihead_attention (src/models.rs:131-176) for one (head, batch column) of a
-// prefill chunk whose cache rows are already written: scores over t = 0..=pos
-// against the kv head h / attn_groups, softmax with max subtraction and
-// division by the sum (:68-81), then the weighted sum of V.
-// Dynamic LDS: att[pos+1].  head_size must be 128.
-__global__ __launch_bounds__(256) void attention_kernel(float *out, const float *q, const float *kcache,
-                                                         const float *vcache, const int32_t *pos,
-                                                         const int32_t *scatter, int n_heads,
-                                                         int n_kv_heads) {
-    constexpr int HS = 128;
-    extern __shared__ float att[];
-    __shared__ float qs[HS];
-    __shared__ float red[16];
-    __shared__ float part[HS];
-    const int h = blockIdx.x, b = blockIdx.y;
-    const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
-    const int p = pos[b];
-    const int kvh = h / (n_heads / n_kv_heads);
-    const int tid = threadIdx.x;
-    if (tid < HS) qs[tid] = q[(size_t)b * dim + h * HS + tid];
-    __syncthreads();
-    const float root = sqrtf((float)HS);
-    // scores: 4 lanes per timestep, 32 dims each
-    const int sub = tid & 3;
-    for (int t = tid >> 2; t <= p; t += 64) {
-        const float4 *kr = reinterpret_cast<const float4 *>(kcache + (size_t)t * kv_dim + kvh * HS + sub * 32);
-        const float4 *qr = reinterpret_cast<const float4 *>(qs + sub * 32);
-        float s = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float4 kk = kr[i], qq = qr[i];
-            s = fmaf(qq.x, kk.x, s);
-            s = fmaf(qq.y, kk.y, s);
-            s = fmaf(qq.z, kk.z, s);
-            s = fmaf(qq.w, kk.w, s);
-        }
-        s += dpp_xchg<0xB1>(s);
-        s += dpp_xchg<0x4E>(s);
-        if (sub == 0) att[t] = s / root;
-    }
-    __syncthreads();
-    float m = -INFINITY;
-    for (int t = tid; t <= p; t += 256) m = fmaxf(m, att[t]);
-    m = block_max(m, red);
-    float sum = 0.f;
-    for (int t = tid; t <= p; t += 256) {
-        const float e = expf(att[t] - m);
-        att[t] = e;
-        sum += e;
-    }
-    sum = block_sum(sum, red);
-    for (int t = tid; t <= p; t += 256) att[t] = att[t] / sum;
-    __syncthreads();
-    // weighted values: thread -> (dim d, parity of t)
-    const int d = tid & (HS - 1), par = tid >> 7;
-    float acc = 0.f;
-#pragma unroll 4
-    for (int t = par; t <= p; t += 2)
-        acc = fmaf(att[t], vcache[(size_t)t * kv_dim + kvh * HS + d], acc);
-    if (par == 1) part[d] = acc;
-    __syncthreads();
-    if (par == 0) {
-        acc += part[d];
-        const int i = h * HS + d;
-        const int dst = scatter ? scatter[i] : i;
-        out[(size_t)b * dim + dst] = acc;
-    }
-}
 
 // Order-preserving key for (value, index): larger value wins, equal values ->
 // larger index wins, which is util::argmax's last-index rule (src/util.rs:39-46).
@@ -366,18 +297,6 @@ int rope_kv_launch(float *q, const float *k, const float *v, const int32_t *pos,
                    int head_size, int B, hipStream_t st) {
     hipLaunchKernelGGL(rope_kv_kernel, dim3(B), dim3(1024), 0, st, q, k, v, pos, cos_t, sin_t, kcache_l,
                        vcache_l, n_heads, n_kv_heads, head_size);
-    L2_HIP(hipGetLastError());
-    return L2_OK;
-}
-
-int attention_launch(float *out, const float *q, const float *kcache_l, const float *vcache_l,
-                     const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
-                     int head_size, int max_pos, int B, hipStream_t st) {
-    if (head_size != 128) return l2_fail(L2_ERR_ARG, "attention: head_size=%d (128 only)", head_size);
-    const size_t lds = (size_t)(max_pos + 1) * sizeof(float);
-    if (lds > 60 * 1024) return l2_fail(L2_ERR_RANGE, "attention: position %d too deep for this kernel", max_pos);
-    hipLaunchKernelGGL(attention_kernel, dim3(n_heads, B), dim3(256), lds, st, out, q, kcache_l, vcache_l,
-                       pos, scatter, n_heads, n_kv_heads);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }

@@ -31,6 +31,7 @@
 // the weight side is none at all; for G = 32 a K step of 64 straddles two
 // groups, and the weights are multiplied by fp16(scale) before the MFMA.
 #include "l2_internal.h"
+#include <algorithm>
 
 namespace {
 
@@ -61,10 +62,23 @@ __device__ __forceinline__ h8 dequant8(uint32_t w, h2 neg_off, h2 scale) {
     return a.v;
 }
 
+template <class T>
+__device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_offset);
+}
+
+// Software pipeline of the K loop.  Everything a K step needs is loaded PW (weights, zeros, scales) or
+// XP (the activation tile) steps ahead, unconditionally (steps past the end of the block's K slice
+// re-read its last step), into rings of registers indexed statically by the position in the loop body,
+// which is unrolled PW times.  Loads return in order, so a wait for the oldest ring slot leaves all the
+// younger ones in flight; with one block of 4 waves on a CU this depth, not occupancy, hides HBM latency.
+constexpr int kGemmPW = 4;
+constexpr int kGemmXP = 2;
+
 template <int G, int NB>
 __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
                                                       float *__restrict__ ws, int KS) {
-    constexpr int MT = 1;
+    constexpr int PW = kGemmPW, XP = kGemmXP;
     constexpr int TN = 32 * NB;
     constexpr bool SA = G >= 64; // scale after the group's partial sum
     extern __shared__ _Float16 xs[]; // [2][TN][kXRow]
@@ -88,178 +102,188 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     const int r = lane & 31, h = lane >> 5;
     const int C4 = in >> 5; // uint4 per weight row
 
-    int orow[MT];
-    bool live[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-        const int o = rb * 128 + wave * 32 + mt * 32 + r;
-        live[mt] = o < n_out;
-        orow[mt] = live[mt] ? o : n_out - 1;
-    }
+    const int o_lane = rb * 128 + wave * 32 + r;
+    const int orow = min(o_lane, n_out - 1);
+    const int grow = min(rb * 128 + (tid & 127), n_out - 1); // the row whose group scale this thread fetches
 
-    f16v acc[MT][NB];  // running result
-    f16v accg[MT][NB]; // partial sum of the current group (SA only)
+    f16v acc[NB];  // running result
+    f16v accg[NB]; // partial sum of the current group (SA only)
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++)
+    for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                acc[mt][nb][i] = 0.f;
-                accg[mt][nb][i] = 0.f;
-            }
+        for (int i = 0; i < 16; i++) {
+            acc[nb][i] = 0.f;
+            accg[nb][i] = 0.f;
+        }
     constexpr int KPG = G / 64 > 0 ? G / 64 : 1; // K iterations per group
-    auto load_group_scales = [&](int g, int buf) {
-        const int o = rb * 128 + tid;
-        if (tid < 128) gsc[buf][tid] = o < n_out ? M.scales[(size_t)o * groups + g] : 0.f;
-    };
     // this block's slice of K, in whole groups
     const int ks = blockIdx.z;
     const int n_grp = n_k / KPG;
     const int kit0 = (int)((long)n_grp * ks / KS) * KPG;
     const int kit1 = (int)((long)n_grp * (ks + 1) / KS) * KPG;
+    const int n_it = kit1 - kit0;
 
+    struct WStage {
+        uint4 w;
+        int32_t z;
+        float s;  // this lane's row, scaled form only
+        float gs; // row `grow`, scale-after form only
+    };
+    const void *qw_base = M.qweight;
+    const void *qz_base = M.qzeros;
+    const void *sc_base = M.scales;
+    auto fetch_w = [&](int kit, WStage &d) {
+        const int kc = min(kit, kit1 - 1);
+        const int g = (kc * 64 + 32 * h) / G;
+        d.w = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc * 2 + h) << 4);
+        d.z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
+        if constexpr (SA) {
+            d.gs = ld_at<float>(sc_base, (uint32_t)(grow * groups + kc / KPG) << 2);
+            d.s = 0.f;
+        } else {
+            d.s = ld_at<float>(sc_base, (uint32_t)(orow * groups + g) << 2);
+            d.gs = 0.f;
+        }
+    };
     // staging map: thread -> (token, 16-byte segment) x (TN*8/256) pieces
     constexpr int PIECES = TN * 8 / 256;
-    uint4 stage[PIECES];
-    auto load_stage = [&](int kit) {
+    struct XStage {
+        uint4 v[PIECES];
+    };
+    uint32_t xoff[PIECES]; // byte offset of this thread's pieces within a K step
+#pragma unroll
+    for (int p = 0; p < PIECES; p++) {
+        const int idx = p * 256 + tid;
+        const int t = idx >> 3, seg = idx & 7;
+        xoff[p] = ((uint32_t)min(t0 + t, B - 1) * (uint32_t)in + seg * 8) * 2u;
+    }
+    auto fetch_x = [&](int kit, XStage &d) {
+        const uint32_t kb = (uint32_t)min(kit, kit1 - 1) * 128u;
+#pragma unroll
+        for (int p = 0; p < PIECES; p++) d.v[p] = ld_at<uint4>(xh, xoff[p] + kb);
+    };
+    auto store_x = [&](int buf, const XStage &d) {
 #pragma unroll
         for (int p = 0; p < PIECES; p++) {
             const int idx = p * 256 + tid;
             const int t = idx >> 3, seg = idx & 7;
-            const int tg = t0 + t;
-            stage[p] = tg < B ? *reinterpret_cast<const uint4 *>(xh + (size_t)tg * in + (size_t)kit * 64 + seg * 8)
-                              : make_uint4(0, 0, 0, 0);
-        }
-    };
-    auto store_stage = [&](int buf) {
-#pragma unroll
-        for (int p = 0; p < PIECES; p++) {
-            const int idx = p * 256 + tid;
-            const int t = idx >> 3, seg = idx & 7;
-            *reinterpret_cast<uint4 *>(xs + ((size_t)buf * TN + t) * kXRow + seg * 8) = stage[p];
+            *reinterpret_cast<uint4 *>(xs + ((size_t)buf * TN + t) * kXRow + seg * 8) = d.v[p];
         }
     };
 
-    uint4 wq[MT];
-    float sc[MT];
-    int32_t zw[MT];
-    auto load_w = [&](int kit) {
-        const int g = (kit * 64 + 32 * h) / G;
+    XStage xr[XP];
+    WStage wr[PW];
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            wq[mt] = M.qweight[(size_t)orow[mt] * C4 + kit * 2 + h];
-            sc[mt] = M.scales[(size_t)orow[mt] * groups + g];
-            zw[mt] = M.qzeros[(size_t)(orow[mt] >> 3) * groups + g];
-        }
-    };
-
-    load_stage(kit0);
-    load_w(kit0);
-    store_stage(0);
-    if (SA) load_group_scales(kit0 / KPG, (kit0 / KPG) & 1);
+    for (int j = 0; j < XP; j++) fetch_x(kit0 + j, xr[j]);
+#pragma unroll
+    for (int j = 0; j < PW; j++) fetch_w(kit0 + j, wr[j]);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the loop's waits then reflect its own order only
+    store_x(0, xr[0]);
+    if (SA && tid < 128) gsc[(kit0 / KPG) & 1][tid] = wr[0].gs;
     __syncthreads();
 
-    for (int kit = kit0; kit < kit1; kit++) {
-        const int buf = (kit - kit0) & 1;
-        // this iteration's weights -> registers of their own, then request the next
-        uint4 wc[MT];
-        h2 noff[MT], s16[MT];
+    for (int base = 0; base < n_it; base += PW) {
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            wc[mt] = wq[mt];
-            const int zn = (zw[mt] >> (4 * (orow[mt] & 7))) & 15;
+        for (int u = 0; u < PW; u++) {
+            if (base + u >= n_it) break; // uniform
+            const int kit = kit0 + base + u;
+            const int buf = (base + u) & 1; // PW is even: the parity of u
+            // this step's weights -> registers of their own, then refill the slot
+            const uint4 wc = wr[u].w;
+            const int zn = (wr[u].z >> (4 * (orow & 7))) & 15;
             const _Float16 off = (_Float16)(-(1024.0f + (float)(zn + 1)));
-            noff[mt] = h2{off, off};
-            const _Float16 s = (_Float16)sc[mt];
-            s16[mt] = h2{s, s};
-        }
-        if (kit + 1 < kit1) {
-            load_stage(kit + 1);
-            load_w(kit + 1);
-        }
-        const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
+            const h2 noff = h2{off, off};
+            const _Float16 s1 = (_Float16)wr[u].s;
+            const h2 s16 = h2{s1, s1};
+            uint32_t w0 = wc.x, w1 = wc.y, w2 = wc.z, w3 = wc.w;
+            asm volatile("" : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3)::"memory");
+            __builtin_amdgcn_sched_barrier(0);
+            fetch_w(kit + PW, wr[u]);
+            fetch_x(kit + XP, xr[u % XP]);
+            __builtin_amdgcn_sched_barrier(0);
+            const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            h8 a[MT];
+            for (int j = 0; j < 4; j++) {
+                const uint32_t word = j == 0 ? w0 : j == 1 ? w1 : j == 2 ? w2 : w3;
+                const h8 a = dequant8<!SA>(word, noff, s16);
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) {
-                const uint32_t word = j == 0 ? wc[mt].x : j == 1 ? wc[mt].y : j == 2 ? wc[mt].z : wc[mt].w;
-                a[mt] = dequant8<!SA>(word, noff[mt], s16[mt]);
-            }
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                const h8 b = *reinterpret_cast<const h8 *>(xb + (size_t)(nb * 32 + r) * kXRow + (4 * h + j) * 8);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
+                for (int nb = 0; nb < NB; nb++) {
+                    const h8 b = *reinterpret_cast<const h8 *>(xb + (size_t)(nb * 32 + r) * kXRow + (4 * h + j) * 8);
                     if (SA)
-                        accg[mt][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, accg[mt][nb], 0, 0, 0);
+                        accg[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, accg[nb], 0, 0, 0);
                     else
-                        acc[mt][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, acc[mt][nb], 0, 0, 0);
+                        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[nb], 0, 0, 0);
                 }
             }
-        }
-        if (SA && (kit + 1) % KPG == 0) {
-            // end of a group: fold its partial sum into the result with the fp32 scale of each row
-            const int gb = (kit / KPG) & 1;
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
+            if (SA && (u + 1) % KPG == 0) {
+                // end of a group: fold its partial sum into the result with the fp32 scale of each row
+                const int gb = (kit / KPG) & 1;
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][wave * 32 + mt * 32 + q * 8 + h * 4]);
+                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][wave * 32 + q * 8 + h * 4]);
                     const float svv[4] = {sv.x, sv.y, sv.z, sv.w};
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++)
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            acc[mt][nb][4 * q + e] = fmaf(svv[e], accg[mt][nb][4 * q + e], acc[mt][nb][4 * q + e]);
-                            accg[mt][nb][4 * q + e] = 0.f;
+                            acc[nb][4 * q + e] = fmaf(svv[e], accg[nb][4 * q + e], acc[nb][4 * q + e]);
+                            accg[nb][4 * q + e] = 0.f;
                         }
                 }
-            if (kit + 1 < kit1) load_group_scales((kit + 1) / KPG, gb ^ 1);
+                // the next group's scales (fetched PW - 1 steps ago with the next step's weights)
+                if (tid < 128) gsc[gb ^ 1][tid] = wr[(u + 1) % PW].gs;
+            }
+            // the next step's activation tile was fetched XP - 1 steps ago
+            store_x(buf ^ 1, xr[(u + 1) % XP]);
+            __syncthreads();
         }
-        if (kit + 1 < kit1) store_stage(buf ^ 1);
-        __syncthreads();
     }
 
-    // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4
+    // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4.
+    // Stored as it stands, every store instruction would touch 64 separate 16-byte pieces; instead each
+    // wave turns its 32 rows x 32 tokens through LDS (the activation buffers are free now) so that a
+    // store instruction writes 8 tokens x 128 contiguous bytes.
     const Q4Epi &E = L.e;
     // workspace of matrix mi starts after those of the matrices before it
     size_t ws_base = 0;
     for (int i = 0; i < mi; i++) ws_base += (size_t)KS * B * L.m[i].out;
+    const int obase = rb * 128 + wave * 32;
+    constexpr int kTRow = 36; // floats per staged token row: 32 + 4 pad (16-byte reads of 8 lanes per token)
+    float *tile = reinterpret_cast<float *>(xs) + wave * 32 * kTRow; // 4.5 KB per wave
+    const int tl = lane >> 3, oc = (lane & 7) * 4; // read-back map: token within a pass of 8, 4 rows
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-        const int obase = rb * 128 + wave * 32 + mt * 32;
-        if (obase >= n_out) continue;
+    for (int nb = 0; nb < NB; nb++) {
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            const int t = t0 + nb * 32 + r;
-            if (t >= B) continue;
+        for (int q = 0; q < 4; q++)
+            *reinterpret_cast<float4 *>(&tile[r * kTRow + q * 8 + h * 4]) =
+                make_float4(acc[nb][4 * q + 0], acc[nb][4 * q + 1], acc[nb][4 * q + 2], acc[nb][4 * q + 3]);
+        // the wave reads what the wave wrote: no block barrier, the LDS queue of a wave is in order
+#pragma unroll
+        for (int pass = 0; pass < 4; pass++) {
+            const int tt = pass * 8 + tl;
+            float4 v = *reinterpret_cast<const float4 *>(&tile[tt * kTRow + oc]);
+            const int t = t0 + nb * 32 + tt;
+            const int o = obase + oc;
+            if (t >= B || o >= n_out) continue;
             const size_t row = (size_t)t * n_out;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int o = obase + q * 8 + h * 4;
-                float4 v = make_float4(acc[mt][nb][4 * q + 0], acc[mt][nb][4 * q + 1], acc[mt][nb][4 * q + 2],
-                                       acc[mt][nb][4 * q + 3]);
-                if (KS > 1) { // partial tile of this K slice
-                    *reinterpret_cast<float4 *>(ws + ws_base + ((size_t)ks * B + t) * n_out + o) = v;
-                    continue;
-                }
-                const float scale_t = ss ? ss[t] : 1.0f;
-                v.x *= scale_t, v.y *= scale_t, v.z *= scale_t, v.w *= scale_t;
-                if (E.kind == Q4_EPI_RESIDUAL) {
-                    const float4 rr = *reinterpret_cast<const float4 *>(E.res + row + o);
-                    v.x += rr.x;
-                    v.y += rr.y;
-                    v.z += rr.z;
-                    v.w += rr.w;
-                }
-                if (E.kind != Q4_EPI_SCATTER_ONLY) *reinterpret_cast<float4 *>(M.y + row + o) = v;
-                const float vals[4] = {v.x, v.y, v.z, v.w};
-                for (int c = 0; c < E.n_scatter; c++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) E.sc_out[c][row + E.sc_idx[c][o + e]] = vals[e];
+            if (KS > 1) { // partial tile of this K slice
+                *reinterpret_cast<float4 *>(ws + ws_base + ((size_t)ks * B + t) * n_out + o) = v;
+                continue;
             }
+            const float scale_t = ss ? ss[t] : 1.0f;
+            v.x *= scale_t, v.y *= scale_t, v.z *= scale_t, v.w *= scale_t;
+            if (E.kind == Q4_EPI_RESIDUAL) {
+                const float4 rr = *reinterpret_cast<const float4 *>(E.res + row + o);
+                v.x += rr.x;
+                v.y += rr.y;
+                v.z += rr.z;
+                v.w += rr.w;
+            }
+            if (E.kind != Q4_EPI_SCATTER_ONLY) *reinterpret_cast<float4 *>(M.y + row + o) = v;
+            const float vals[4] = {v.x, v.y, v.z, v.w};
+            for (int c = 0; c < E.n_scatter; c++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) E.sc_out[c][row + E.sc_idx[c][o + e]] = vals[e];
         }
     }
 }
@@ -292,7 +316,10 @@ __global__ __launch_bounds__(256) void q4_gemm_reduce_kernel(const Q4Launch L, c
 
 // fp32 [B][n] (already in the consumer's g_index order) -> fp16 [B][n], times the
 // norm weight if given, with the (0,4,1,5,2,6,3,7) interleave inside every 8.
-__global__ void prep_f16_kernel(_Float16 *out, const float *x, const float *wn, int n) {
+__global__ void prep_f16_kernel(const PrepList P, int n) {
+    _Float16 *out = reinterpret_cast<_Float16 *>(P.out[blockIdx.z]);
+    const float *x = P.x[blockIdx.z];
+    const float *wn = P.wn[blockIdx.z];
     const int b = blockIdx.y;
     const int j8 = blockIdx.x * blockDim.x + threadIdx.x; // group of 8
     if (j8 * 8 >= n) return;
@@ -335,14 +362,19 @@ __global__ __launch_bounds__(256) void rms_scale_kernel(float *ss, const float *
 }
 
 // silu gate (src/models.rs:92-98) for a chunk: out[b][scatter[i]] = silu(a[b][i]) * c[b][i]
-__global__ void silu_scatter_kernel(float *out, const float *a, const float *c, const int32_t *scatter, int n) {
+__global__ void silu_scatter_kernel(float *out, _Float16 *out_h, const float *a, const float *c,
+                                    const int32_t *scatter, int n) {
     const int b = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float s = a[(size_t)b * n + i];
     s = s * (1.0f / (1.0f + expf(-s)));
     s = s * c[(size_t)b * n + i];
-    out[(size_t)b * n + (scatter ? scatter[i] : i)] = s;
+    const int j = scatter ? scatter[i] : i;
+    if (out_h)
+        out_h[(size_t)b * n + h16_slot(j)] = (_Float16)s;
+    else
+        out[(size_t)b * n + j] = s;
 }
 
 template <int G>
@@ -355,7 +387,10 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
         rows += L.m[i].out;
     }
     const int B = L.batch;
-    const int NB = B > 64 ? 4 : B > 32 ? 2 : 1;
+    // 64 tokens per block even for longer chunks: 128 would halve the weight traffic, but its 128
+    // accumulator registers leave one block per CU, and the K loop (a barrier every 64 k) then has nothing
+    // to overlap with (measured: w1|w3 of 7B at 128 tokens 73 us, at 2 x 64 tokens 52 us).
+    const int NB = B > 32 ? 2 : 1;
     const int TN = 32 * NB;
     const int t_tiles = (B + TN - 1) / TN;
     // K slices: aim at ~2 blocks per CU, whole groups per slice, at most 8
@@ -366,11 +401,12 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     if (KS < 1) KS = 1;
     while (KS > 1 && (size_t)KS * B * rows > ws_floats) KS--;
     dim3 grid(total, t_tiles, KS), block(256);
-    const size_t lds = (size_t)2 * TN * kXRow * sizeof(_Float16);
+    // the activation buffers, or the four output staging tiles of the epilogue (32 x 36 floats per wave)
+    const size_t lds = std::max((size_t)2 * TN * kXRow * sizeof(_Float16), (size_t)4 * 32 * 36 * sizeof(float));
     switch (NB) {
         case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1>), grid, block, lds, st, L, xh, ss, ws, KS); break;
         case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2>), grid, block, lds, st, L, xh, ss, ws, KS); break;
-        default: hipLaunchKernelGGL((q4_gemm_kernel<G, 4>), grid, block, lds, st, L, xh, ss, ws, KS); break;
+        default: return l2_fail(L2_ERR_ARG, "q4 gemm: token tile");
     }
     L2_HIP(hipGetLastError());
     if (KS > 1) {
@@ -399,11 +435,17 @@ int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, floa
 
 bool q4_gemm_supports(int in, int out) { return in % 64 == 0 && out % 32 == 0; }
 
-int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st) {
-    if (n % 8) return l2_fail(L2_ERR_ARG, "prep: n=%d not a multiple of 8", n);
-    hipLaunchKernelGGL(prep_f16_kernel, dim3((n / 8 + 255) / 256, B), dim3(256), 0, st, (_Float16 *)out_f16, x, wn, n);
+int prep_f16_multi_launch(const PrepList &P, int n, int B, hipStream_t st) {
+    if (n % 8 || P.n_mats < 1 || P.n_mats > 3) return l2_fail(L2_ERR_ARG, "prep: n=%d, %d vectors", n, P.n_mats);
+    hipLaunchKernelGGL(prep_f16_kernel, dim3((n / 8 + 255) / 256, B, P.n_mats), dim3(256), 0, st, P, n);
     L2_HIP(hipGetLastError());
     return L2_OK;
+}
+
+int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st) {
+    PrepList P{};
+    P.out[0] = out_f16, P.x[0] = x, P.wn[0] = wn, P.n_mats = 1;
+    return prep_f16_multi_launch(P, n, B, st);
 }
 
 int rms_scale_launch(float *ss, const float *x, float eps, int dim, int B, hipStream_t st) {
@@ -412,9 +454,10 @@ int rms_scale_launch(float *ss, const float *x, float eps, int dim, int B, hipSt
     return L2_OK;
 }
 
-int silu_scatter_launch(float *out, const float *a, const float *c, const int32_t *scatter, int n, int B,
-                        hipStream_t st) {
-    hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, a, c, scatter, n);
+int silu_scatter_launch(float *out, void *out_f16, const float *a, const float *c, const int32_t *scatter, int n,
+                        int B, hipStream_t st) {
+    hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, (_Float16 *)out_f16, a, c,
+                       scatter, n);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }

@@ -111,9 +111,24 @@ int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, float *ws, si
 bool q4_gemm_supports(int in, int out);
 // out_f16[b][j'] = fp16(x[b][j] * (wn ? wn[j] : 1)), j' = j with the order (0,4,1,5,2,6,3,7) inside every 8.
 int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st);
+// The same for up to three vectors of one length in one launch (q|k|v, w1|w3 inputs).
+struct PrepList {
+    void *out[3];
+    const float *x[3];
+    const float *wn[3];
+    int n_mats;
+};
+int prep_f16_multi_launch(const PrepList &P, int n, int B, hipStream_t st);
 int rms_scale_launch(float *ss, const float *x, float eps, int dim, int B, hipStream_t st);
-int silu_scatter_launch(float *out, const float *a, const float *c, const int32_t *scatter, int n, int B,
-                        hipStream_t st);
+// out[b][scatter[i]] = silu(a[b][i]) * c[b][i]; with out_f16 set the result goes there instead, as fp16 in
+// the pair-interleaved order the GEMM reads (no separate conversion pass).
+int silu_scatter_launch(float *out, void *out_f16, const float *a, const float *c, const int32_t *scatter, int n,
+                        int B, hipStream_t st);
+// Slot of element j of a vector in the fp16 pair-interleaved order: (0,4,1,5,2,6,3,7) inside every 8.
+__host__ __device__ inline int h16_slot(int j) {
+    const int e = j & 7;
+    return (j & ~7) | (e < 4 ? 2 * e : 2 * (e - 4) + 1);
+}
 
 // ---- the other per-token kernels -------------------------------------------
 
@@ -131,7 +146,7 @@ int rope_kv_launch(float *q, const float *k, const float *v, const int32_t *pos,
                    const float *sin_t, float *kcache_l, float *vcache_l, int n_heads, int n_kv_heads,
                    int head_size, int B, hipStream_t st);
 // Batched attention over an already written cache: out[b][scatter[i]] for query b at pos[b].
-int attention_launch(float *out, const float *q, const float *kcache_l, const float *vcache_l,
+int attention_launch(float *out, void *out_f16, const float *q, const float *kcache_l, const float *vcache_l,
                      const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
                      int head_size, int max_pos, int B, hipStream_t st);
 
