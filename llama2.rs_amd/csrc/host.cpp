@@ -398,7 +398,12 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
         return l2_fail(L2_ERR_FORMAT, "weights are %zu bytes, the struct for these dims is %zu", nbytes,
                        l2_weights_bytes(dims));
     if (max_seq <= 0) max_seq = dims->seq_len;
-    if (max_seq > 15000) return l2_fail(L2_ERR_RANGE, "max_seq %d (at most 15000)", max_seq);
+    {   // the attention kernels address one layer's cache with 32-bit byte offsets
+        const size_t layer_bytes = (size_t)max_seq * dims->n_kv_heads * (dims->dim / dims->n_heads) * 4;
+        if (layer_bytes >= ((size_t)1 << 32))
+            return l2_fail(L2_ERR_RANGE, "max_seq %d: one layer of the cache would be %zu bytes (below 4 GiB)", max_seq,
+                           layer_bytes);
+    }
     L2_TRY(require_device());
 
     l2_model *m = new l2_model();
