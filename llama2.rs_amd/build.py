@@ -25,7 +25,8 @@ SOURCES = {
     # file: extra flags
     "kernels_q4.hip": [],
     "kernels_q4_stream.hip": [],
-    "kernels_q4_gemm.hip": [],
+    # MFMA accumulators in VGPRs: the per-group fold reads and writes them with plain FMAs
+    "kernels_q4_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     # the block kernels keep the reference's rounded-multiply-then-add where they restate it
     "kernels_misc.hip": ["-ffp-contract=off"],
     "kernels_attn.hip": ["-ffp-contract=off"],

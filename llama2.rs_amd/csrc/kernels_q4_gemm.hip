@@ -39,7 +39,7 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int kXRow = 72; // halves per staged token row: 64 + 8 pad
+constexpr int kXPad = 8; // halves of padding per staged token row (K step + 8: 16-byte reads stay conflict-free)
 
 union A8 {
     h8 v;
@@ -47,20 +47,51 @@ union A8 {
     uint32_t u[4];
 };
 
-// One packed word of 8 nibbles -> 8 fp16 values n - z1 (exact), times `scale` if
-// SCALED, in the pair order (0,4,1,5,2,6,3,7).
+// (x & mask) | magic in one instruction; the compiler splits it into v_and + v_or because both constants
+// would be literals.  mask lives in a VGPR, magic in an SGPR (one scalar operand per VALU instruction).
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask_v, uint32_t magic_s) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(mask_v), "s"(magic_s));
+    return r;
+}
+
+struct DequantConsts {
+    uint32_t mask_lo, mask_hi; // 0x000F000F, 0x00F000F0 (VGPRs)
+    uint32_t magic;            // 0x64006400: fp16 1024 in both halves (SGPR)
+    h2 neg_off;                // -(1024 + z1)
+    h2 neg_off16;              // -(64 + z1)
+    h2 sixteenth;              // 1/16
+};
+
+// One packed word of 8 nibbles -> 8 fp16 values n - z1 (exact), times `scale` if SCALED, in the pair
+// order (0,4,1,5,2,6,3,7).  Nibbles 0 and 4 (and 2, 6 after one shift by 8) land in the low mantissa bits
+// of the fp16 pair: 1024 + n.  Nibbles 1 and 5 (3, 7) are taken where they stand, four bits higher:
+// 1024 + 16 n, and one packed FMA with 1/16 brings them to 64 + n, both exact.  9 instructions per word.
 template <bool SCALED>
-__device__ __forceinline__ h8 dequant8(uint32_t w, h2 neg_off, h2 scale) {
+__device__ __forceinline__ h8 dequant8(uint32_t w, const DequantConsts &c, h2 scale) {
     A8 a;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t t = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-        h2 v = __builtin_bit_cast(h2, t);
-        v = v + neg_off; // (1024 + n) - (1024 + z1), exact
-        a.p[i] = SCALED ? v * scale : v;
-    }
+    const uint32_t w8 = w >> 8;
+    h2 v0 = __builtin_bit_cast(h2, and_or(w, c.mask_lo, c.magic)) + c.neg_off;
+    h2 v1 = __builtin_elementwise_fma(__builtin_bit_cast(h2, and_or(w, c.mask_hi, c.magic)), c.sixteenth, c.neg_off16);
+    h2 v2 = __builtin_bit_cast(h2, and_or(w8, c.mask_lo, c.magic)) + c.neg_off;
+    h2 v3 = __builtin_elementwise_fma(__builtin_bit_cast(h2, and_or(w8, c.mask_hi, c.magic)), c.sixteenth, c.neg_off16);
+    a.p[0] = SCALED ? v0 * scale : v0;
+    a.p[1] = SCALED ? v1 * scale : v1;
+    a.p[2] = SCALED ? v2 * scale : v2;
+    a.p[3] = SCALED ? v3 * scale : v3;
     return a.v;
 }
+
+#if defined(Q4G_TS) // measurement build only: per-block timestamps (100 MHz counter)
+__device__ unsigned long long q4g_ts[4096 * 4];
+#define Q4G_STAMP(k)                                                                                    \
+    do {                                                                                                \
+        const unsigned bid_ = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);          \
+        if (threadIdx.x == 0 && bid_ < 4096) q4g_ts[bid_ * 4 + (k)] = wall_clock64();                  \
+    } while (0)
+#else
+#define Q4G_STAMP(k)
+#endif
 
 template <class T>
 __device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
@@ -75,16 +106,20 @@ __device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
 constexpr int kGemmPW = 4;
 constexpr int kGemmXP = 2;
 
-template <int G, int NB>
+template <int G, int NB, int KSTEP>
 __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
                                                       float *__restrict__ ws, int KS) {
+    Q4G_STAMP(0);
     constexpr int PW = kGemmPW, XP = kGemmXP;
+    constexpr int W = KSTEP / 64;        // sub-steps of 64 k per K step
+    constexpr int kXRow = KSTEP + kXPad; // halves per staged token row
+    static_assert(KSTEP == 64 || G >= KSTEP, "a longer K step stays inside one group");
     constexpr int TN = 32 * NB;
     constexpr bool SA = G >= 64; // scale after the group's partial sum
     extern __shared__ _Float16 xs[]; // [2][TN][kXRow]
     __shared__ float gsc[2][128];    // fp32 scales of the block's 128 rows for the current group
     const int in = L.in;
-    const int n_k = in >> 6; // K iterations of 64
+    const int n_k = in / KSTEP; // K iterations
 
     int rb = blockIdx.x;
     int mi = 0;
@@ -115,7 +150,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             acc[nb][i] = 0.f;
             accg[nb][i] = 0.f;
         }
-    constexpr int KPG = G / 64 > 0 ? G / 64 : 1; // K iterations per group
+    constexpr int KPG = G / KSTEP > 0 ? G / KSTEP : 1; // K iterations per group
     // this block's slice of K, in whole groups
     const int ks = blockIdx.z;
     const int n_grp = n_k / KPG;
@@ -124,7 +159,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     const int n_it = kit1 - kit0;
 
     struct WStage {
-        uint4 w;
+        uint4 w[W];
         int32_t z;
         float s;  // this lane's row, scaled form only
         float gs; // row `grow`, scale-after form only
@@ -134,8 +169,10 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     const void *sc_base = M.scales;
     auto fetch_w = [&](int kit, WStage &d) {
         const int kc = min(kit, kit1 - 1);
-        const int g = (kc * 64 + 32 * h) / G;
-        d.w = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc * 2 + h) << 4);
+        const int g = (kc * KSTEP + 32 * h) / G;
+#pragma unroll
+        for (int sw = 0; sw < W; sw++)
+            d.w[sw] = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc * (2 * W) + 2 * sw + h) << 4);
         d.z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
         if constexpr (SA) {
             d.gs = ld_at<float>(sc_base, (uint32_t)(grow * groups + kc / KPG) << 2);
@@ -146,7 +183,8 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
         }
     };
     // staging map: thread -> (token, 16-byte segment) x (TN*8/256) pieces
-    constexpr int PIECES = TN * 8 / 256;
+    constexpr int SEGS = KSTEP / 8; // 16-byte segments per token and K step
+    constexpr int PIECES = TN * SEGS / 256;
     struct XStage {
         uint4 v[PIECES];
     };
@@ -154,11 +192,11 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
 #pragma unroll
     for (int p = 0; p < PIECES; p++) {
         const int idx = p * 256 + tid;
-        const int t = idx >> 3, seg = idx & 7;
+        const int t = idx / SEGS, seg = idx % SEGS;
         xoff[p] = ((uint32_t)min(t0 + t, B - 1) * (uint32_t)in + seg * 8) * 2u;
     }
     auto fetch_x = [&](int kit, XStage &d) {
-        const uint32_t kb = (uint32_t)min(kit, kit1 - 1) * 128u;
+        const uint32_t kb = (uint32_t)min(kit, kit1 - 1) * (uint32_t)(KSTEP * 2);
 #pragma unroll
         for (int p = 0; p < PIECES; p++) d.v[p] = ld_at<uint4>(xh, xoff[p] + kb);
     };
@@ -166,7 +204,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
 #pragma unroll
         for (int p = 0; p < PIECES; p++) {
             const int idx = p * 256 + tid;
-            const int t = idx >> 3, seg = idx & 7;
+            const int t = idx / SEGS, seg = idx % SEGS;
             *reinterpret_cast<uint4 *>(xs + ((size_t)buf * TN + t) * kXRow + seg * 8) = d.v[p];
         }
     };
@@ -181,6 +219,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     store_x(0, xr[0]);
     if (SA && tid < 128) gsc[(kit0 / KPG) & 1][tid] = wr[0].gs;
     __syncthreads();
+    Q4G_STAMP(1);
 
     for (int base = 0; base < n_it; base += PW) {
 #pragma unroll
@@ -189,31 +228,52 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             const int kit = kit0 + base + u;
             const int buf = (base + u) & 1; // PW is even: the parity of u
             // this step's weights -> registers of their own, then refill the slot
-            const uint4 wc = wr[u].w;
             const int zn = (wr[u].z >> (4 * (orow & 7))) & 15;
+            DequantConsts dc;
+            dc.mask_lo = 0x000F000Fu, dc.mask_hi = 0x00F000F0u, dc.magic = 0x64006400u;
             const _Float16 off = (_Float16)(-(1024.0f + (float)(zn + 1)));
-            const h2 noff = h2{off, off};
+            const _Float16 off16 = (_Float16)(-(64.0f + (float)(zn + 1)));
+            dc.neg_off = h2{off, off};
+            dc.neg_off16 = h2{off16, off16};
+            dc.sixteenth = h2{(_Float16)0.0625f, (_Float16)0.0625f};
             const _Float16 s1 = (_Float16)wr[u].s;
             const h2 s16 = h2{s1, s1};
-            uint32_t w0 = wc.x, w1 = wc.y, w2 = wc.z, w3 = wc.w;
-            asm volatile("" : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3)::"memory");
+            uint32_t wd[W][4];
+#pragma unroll
+            for (int sw = 0; sw < W; sw++) {
+                wd[sw][0] = wr[u].w[sw].x, wd[sw][1] = wr[u].w[sw].y, wd[sw][2] = wr[u].w[sw].z, wd[sw][3] = wr[u].w[sw].w;
+                asm volatile("" : "+v"(wd[sw][0]), "+v"(wd[sw][1]), "+v"(wd[sw][2]), "+v"(wd[sw][3])::"memory");
+            }
             __builtin_amdgcn_sched_barrier(0);
             fetch_w(kit + PW, wr[u]);
             fetch_x(kit + XP, xr[u % XP]);
             __builtin_amdgcn_sched_barrier(0);
             const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
+            // W * 4 steps of 16 k.  The operands of step i + 1 (two LDS reads per token tile, the
+            // dequantised weights) are produced while the MFMAs of step i run: without this the
+            // LDS latency stands in front of every MFMA.
+            constexpr int NSTEP = W * 4;
+            h8 aq[2], bq[2][NB];
+            auto produce = [&](int step, int slot) {
+                const int sw = step >> 2, j = step & 3;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint32_t word = j == 0 ? w0 : j == 1 ? w1 : j == 2 ? w2 : w3;
-                const h8 a = dequant8<!SA>(word, noff, s16);
+                for (int nb = 0; nb < NB; nb++)
+                    bq[slot][nb] = *reinterpret_cast<const h8 *>(xb + (size_t)(nb * 32 + r) * kXRow +
+                                                                 (sw * 8 + 4 * h + j) * 8);
+                aq[slot] = dequant8<!SA>(wd[sw][j], dc, s16);
+            };
+            produce(0, 0);
+#pragma unroll
+            for (int step = 0; step < NSTEP; step++) {
+                if (step + 1 < NSTEP) produce(step + 1, (step + 1) & 1);
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
-                    const h8 b = *reinterpret_cast<const h8 *>(xb + (size_t)(nb * 32 + r) * kXRow + (4 * h + j) * 8);
                     if (SA)
-                        accg[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, accg[nb], 0, 0, 0);
+                        accg[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[step & 1], bq[step & 1][nb], accg[nb], 0, 0, 0);
                     else
-                        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[nb], 0, 0, 0);
+                        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[step & 1], bq[step & 1][nb], acc[nb], 0, 0, 0);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
             if (SA && (u + 1) % KPG == 0) {
                 // end of a group: fold its partial sum into the result with the fp32 scale of each row
@@ -239,6 +299,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
         }
     }
 
+    Q4G_STAMP(2);
     // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4.
     // Stored as it stands, every store instruction would touch 64 separate 16-byte pieces; instead each
     // wave turns its 32 rows x 32 tokens through LDS (the activation buffers are free now) so that a
@@ -286,7 +347,16 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                 for (int e = 0; e < 4; e++) E.sc_out[c][row + E.sc_idx[c][o + e]] = vals[e];
         }
     }
+    Q4G_STAMP(3);
 }
+
+#if defined(Q4G_TS)
+} // namespace
+extern "C" int l2_debug_gemm_ts(unsigned long long *out, int n) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(q4g_ts), (size_t)n * 8);
+}
+namespace {
+#endif
 
 // Adds the KS partial tiles of a split-K GEMM in slice order and runs the epilogue.
 // grid: (ceil(sum_out / 256), B); the matrices of the launch are laid end to end.
@@ -394,7 +464,9 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     const int TN = 32 * NB;
     const int t_tiles = (B + TN - 1) / TN;
     // K slices: aim at ~2 blocks per CU, whole groups per slice, at most 8
-    const int n_grp = (L.in / 64) / (G / 64 > 0 ? G / 64 : 1);
+    // K step: 128 where a group is at least that long (half the block barriers per k), else 64
+    constexpr int KSTEP = G >= 128 ? 128 : 64;
+    const int n_grp = (L.in / KSTEP) / (G / KSTEP > 0 ? G / KSTEP : 1);
     int KS = (512 + total * t_tiles - 1) / (total * t_tiles);
     if (KS > 8) KS = 8;
     if (KS > n_grp) KS = n_grp;
@@ -402,10 +474,10 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     while (KS > 1 && (size_t)KS * B * rows > ws_floats) KS--;
     dim3 grid(total, t_tiles, KS), block(256);
     // the activation buffers, or the four output staging tiles of the epilogue (32 x 36 floats per wave)
-    const size_t lds = std::max((size_t)2 * TN * kXRow * sizeof(_Float16), (size_t)4 * 32 * 36 * sizeof(float));
+    const size_t lds = std::max((size_t)2 * TN * (KSTEP + kXPad) * sizeof(_Float16), (size_t)4 * 32 * 36 * sizeof(float));
     switch (NB) {
-        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1>), grid, block, lds, st, L, xh, ss, ws, KS); break;
-        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2>), grid, block, lds, st, L, xh, ss, ws, KS); break;
+        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS); break;
+        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS); break;
         default: return l2_fail(L2_ERR_ARG, "q4 gemm: token tile");
     }
     L2_HIP(hipGetLastError());
@@ -421,7 +493,7 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
 int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, float *ws, size_t ws_floats,
                    hipStream_t st) {
     if (L.n_mats < 1 || L.n_mats > 3) return l2_fail(L2_ERR_ARG, "q4 gemm: n_mats=%d", L.n_mats);
-    if (L.in % 64 != 0 || L.in % L.group_size != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d must be a multiple of 64", L.in);
+    if (L.in % 128 != 0 || L.in % L.group_size != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d must be a multiple of 128", L.in);
     for (int i = 0; i < L.n_mats; i++)
         if (L.m[i].out % 32 != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: out=%d must be a multiple of 32", L.m[i].out);
     if (L.pair) return l2_fail(L2_ERR_ARG, "q4 gemm: pair launches are not supported");
@@ -433,7 +505,7 @@ int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, floa
     return l2_fail(L2_ERR_ARG, "q4 gemm: group size %d", L.group_size);
 }
 
-bool q4_gemm_supports(int in, int out) { return in % 64 == 0 && out % 32 == 0; }
+bool q4_gemm_supports(int in, int out) { return in % 128 == 0 && out % 32 == 0; }
 
 int prep_f16_multi_launch(const PrepList &P, int n, int B, hipStream_t st) {
     if (n % 8 || P.n_mats < 1 || P.n_mats > 3) return l2_fail(L2_ERR_ARG, "prep: n=%d, %d vectors", n, P.n_mats);
