@@ -57,7 +57,8 @@ typedef struct l2_dims {
     int32_t n_kv_heads;
     int32_t vocab_size;
     int32_t seq_len;    /* rows of the deprecated freq tables stored in the file (2048) */
-    int32_t group_size; /* 32, 64 or 128 */
+    int32_t group_size; /* 32, 64 or 128; 0 = the model without quantisation (GROUPSIZE 0, src/constants.rs:58-61):
+                         * TransformerWeights, every projection a dense [OUT][IN] fp32 matrix (src/model.rs:36-67) */
 } l2_dims;
 
 /* Config as read from the 28-byte header (src/constants.rs:80-89, 102-119). */

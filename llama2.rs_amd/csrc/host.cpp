@@ -42,6 +42,7 @@ extern "C" const char *l2_last_error(void) { return g_err; }
 static int64_t div_up(int64_t x, int64_t y) { return x / y + (x % y == 0 ? 0 : 1); }
 
 static size_t qlinear_bytes(int in, int out, int g) {
+    if (g == 0) return (size_t)out * in * 4; // dense Linear<IN,OUT> (src/model.rs:11-15)
     const size_t groups = (size_t)div_up(in, g);
     return (size_t)out * (in / 8) * 4 + (size_t)(out / 8) * groups * 4 + (size_t)out * groups * 4 +
            (size_t)in * 4;
@@ -52,13 +53,16 @@ static int check_dims(const l2_dims *d) {
     if (d->dim <= 0 || d->hidden_dim <= 0 || d->n_layers <= 0 || d->n_heads <= 0 ||
         d->n_kv_heads <= 0 || d->vocab_size <= 0 || d->seq_len <= 0)
         return l2_fail(L2_ERR_ARG, "dims: non-positive field");
-    if (d->group_size != 32 && d->group_size != 64 && d->group_size != 128)
-        return l2_fail(L2_ERR_ARG, "dims: group_size %d (32, 64 or 128)", d->group_size);
+    // 0 is the build without quantisation (GROUPSIZE of src/constants.rs:58-61): every projection dense
+    if (d->group_size != 0 && d->group_size != 32 && d->group_size != 64 && d->group_size != 128)
+        return l2_fail(L2_ERR_ARG, "dims: group_size %d (32, 64, 128, or 0 for the model without quantisation)",
+                       d->group_size);
     if (d->dim % d->n_heads || d->n_heads % d->n_kv_heads)
         return l2_fail(L2_ERR_ARG, "dims: heads do not divide");
     if (d->dim / d->n_heads != 128)
         return l2_fail(L2_ERR_ARG, "dims: head size %d (the kernels are built for 128)", d->dim / d->n_heads);
-    if (d->dim % d->group_size || d->hidden_dim % d->group_size || d->dim % 32 || d->hidden_dim % 32)
+    if ((d->group_size && (d->dim % d->group_size || d->hidden_dim % d->group_size)) || d->dim % 32 ||
+        d->hidden_dim % 32)
         return l2_fail(L2_ERR_ARG, "dims: dim and hidden_dim must be multiples of 32 and of the group size");
     return L2_OK;
 }
@@ -205,6 +209,10 @@ struct Walker {
     }
     void qlinears(int in, int out) {
         const int G = d.group_size;
+        if (G == 0) { // dense projections, N(0, 0.02) like the embedding
+            for (int l = 0; l < d.n_layers; l++) add(2, (size_t)out * in);
+            return;
+        }
         const size_t groups = (size_t)div_up(in, G);
         for (int l = 0; l < d.n_layers; l++) {
             add(0, (size_t)out * (in / 8));
@@ -280,7 +288,8 @@ struct l2_model {
     // the raw residual stream in the input order of the named projection.
     int cap_B = 0;
     float *x = nullptr, *xq = nullptr, *xk = nullptr, *xv = nullptr, *qv = nullptr, *kv = nullptr,
-          *vv = nullptr, *attg = nullptr, *x1 = nullptr, *x3 = nullptr, *hg = nullptr, *logits = nullptr;
+          *vv = nullptr, *attg = nullptr, *x1 = nullptr, *x3 = nullptr, *hg = nullptr, *hd = nullptr,
+          *logits = nullptr;
     // extra scratch of the MFMA prefill path (cap_B_mfma columns): fp16 inputs, w1/w3 outputs, row scales
     int cap_B_mfma = 0;
     void *h16a = nullptr, *h16b = nullptr, *h16c = nullptr; // fp16 [B][max(dim, hidden)]
@@ -313,7 +322,7 @@ static constexpr int kMaxSplits = 64;
             l2_model::ProfRec r_{cls_, nullptr, nullptr};                           \
             L2_HIP(hipEventCreate(&r_.e0));                                         \
             L2_HIP(hipEventCreate(&r_.e1));                                         \
-            const bool q4_ = (cls_) == K_Q4_QKV || (cls_) == K_Q4_WO || (cls_) == K_Q4_W13 || (cls_) == K_Q4_W2; \
+            const bool q4_ = m->d.group_size != 0 && ((cls_) == K_Q4_QKV || (cls_) == K_Q4_WO || (cls_) == K_Q4_W13 || (cls_) == K_Q4_W2); \
             if (q4_) {                                                              \
                 g_q4_prof.start = r_.e0;                                            \
                 g_q4_prof.stop = r_.e1;                                             \
@@ -452,8 +461,18 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
     struct Pending { int proj, layer; size_t host_off; int in; size_t inv_off; };
     std::vector<Pending> pend;
     auto qblock = [&](int proj, int in, int outn) {
-        const int groups = (int)div_up(in, G);
         m->q[proj].resize(L);
+        if (G == 0) { // src/model.rs:36-67: the same field order, every projection a dense matrix
+            for (int l = 0; l < L; l++) {
+                DevQLinear &q = m->q[proj][l];
+                q.in = in;
+                q.out = outn;
+                q.dense = (const float *)(dbase + off);
+                off += (size_t)outn * in * 4;
+            }
+            return;
+        }
+        const int groups = (int)div_up(in, G);
         for (int l = 0; l < L; l++) {
             DevQLinear &q = m->q[proj][l];
             q.in = in;
@@ -488,7 +507,7 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
     if (off != nbytes) return bail(l2_fail(L2_ERR_FORMAT, "internal: walked %zu of %zu bytes", off, nbytes));
 
     // inverse act-order permutations (also validates every g_index)
-    {
+    if (G != 0) {
         std::vector<int32_t> inv(inv_total);
         bool ok = true;
         for (const Pending &p : pend) {
@@ -502,9 +521,10 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
         for (const Pending &p : pend) m->q[p.proj][p.layer].inv_index = m->dinv + p.inv_off;
     }
 
+    M_TRY(dalloc(&m->attn_part, (size_t)dims->n_heads * kMaxSplits * 130));
     // Norm weights re-ordered for each consumer of a normalised vector, so that the
     // matvec prologue reads them linearly: wn_c[j] = w[g_index_c[j]].
-    {
+    if (G != 0) {
         const size_t per_layer = (size_t)5 * dim;
         std::vector<float> wn((size_t)L * per_layer);
         const float *att_h = (const float *)(weights + ((const char *)m->rms_att - dbase));
@@ -519,7 +539,6 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
             }
         M_TRY(dalloc(&m->dwn, wn.size()));
         M_HIP(hipMemcpy(m->dwn, wn.data(), wn.size() * 4, hipMemcpyHostToDevice));
-        M_TRY(dalloc(&m->attn_part, (size_t)dims->n_heads * kMaxSplits * 130));
     }
 
     // RoPE angles exactly as the reference evaluates them per element
@@ -601,7 +620,7 @@ extern "C" void l2_model_close(l2_model *m) {
     if (!m) return;
     if (m->stream) (void)hipStreamSynchronize(m->stream);
     void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->dwn, m->attn_part, m->x, m->xq, m->xk,
-                    m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->logits, m->dtok, m->dpos,
+                    m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->hd, m->logits, m->dtok, m->dpos,
                     m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y, m->h16a, m->h16b, m->h16c,
                     m->hb, m->hb2, m->ssb, m->gemm_ws};
     for (void *p : ptrs) dfree(p);
@@ -628,6 +647,8 @@ extern "C" int l2_prefill_supported(const l2_model *m) { return m ? 1 : 0; }
 extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
     if (!m) return l2_fail(L2_ERR_ARG, "null model");
     if (mode != L2_PREFILL_FP32 && mode != L2_PREFILL_MFMA) return l2_fail(L2_ERR_ARG, "prefill mode %d", mode);
+    if (mode == L2_PREFILL_MFMA && m->d.group_size == 0)
+        return l2_fail(L2_ERR_ARG, "the MFMA prefill path is the quantised model's");
     if (mode == L2_PREFILL_MFMA && !(q4_gemm_supports(m->d.dim, m->d.dim) && q4_gemm_supports(m->d.hidden_dim, m->kv_dim) &&
                                      q4_gemm_supports(m->d.dim, m->d.hidden_dim)))
         return l2_fail(L2_ERR_ARG, "the MFMA prefill path needs dim and hidden_dim to be multiples of 64");
@@ -661,6 +682,11 @@ static int ensure_batch(l2_model *m, int B) {
     L2_TRY(dalloc(&m->x1, B * dim));
     L2_TRY(dalloc(&m->x3, B * dim));
     L2_TRY(dalloc(&m->hg, B * hid));
+    if (m->d.group_size == 0) { // the dense model keeps w1's output beside the gated product
+        dfree(m->hd);
+        m->hd = nullptr;
+        L2_TRY(dalloc(&m->hd, B * hid));
+    }
     L2_TRY(dalloc(&m->dtok, (size_t)B));
     L2_TRY(dalloc(&m->dpos, (size_t)B));
     if (!m->logits) L2_TRY(dalloc(&m->logits, (size_t)m->d.vocab_size));
@@ -892,6 +918,16 @@ extern "C" int l2_model_qmatvec(l2_model *m, int layer, int proj, const float *x
     if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
     const DevQLinear &q = m->q[proj][layer];
     L2_TRY(op_scratch(m, (size_t)B * std::max(std::max(q.in, q.out), m->d.vocab_size)));
+    if (q.dense) { // Linear::matvec<B> (src/model.rs:22-31)
+        hipStream_t st = m->stream;
+        L2_HIP(hipMemcpyAsync(m->op_x, x_host, (size_t)B * q.in * 4, hipMemcpyHostToDevice, st));
+        DenseArgs a{};
+        a.y = m->op_y, a.w = q.dense, a.x = m->op_x, a.in = q.in, a.out = q.out, a.batch = B;
+        L2_TRY(dense_launch(a, st));
+        L2_HIP(hipMemcpyAsync(y_host, m->op_y, (size_t)B * q.out * 4, hipMemcpyDeviceToHost, st));
+        L2_HIP(hipStreamSynchronize(st));
+        return L2_OK;
+    }
     if (B > 1 && m->prefill_mode == L2_PREFILL_MFMA && q4_gemm_supports(q.in, q.out)) {
         // the prefill form of the same operator: gather, round to fp16, dequant -> MFMA
         hipStream_t st = m->stream;
@@ -923,6 +959,22 @@ extern "C" int l2_model_classifier(l2_model *m, const float *x_host, float *y_ho
 // ---------------------------------------------------------------------------
 // transformer<B>
 
+// How the timesteps of a decode step are cut across blocks: one block per kv head up to 256 timesteps,
+// beyond that two blocks per CU where the context allows it, at least 64 timesteps each.
+static void attn_split_policy(int n_t, int n_kv_heads, int *ts_out, int *n_splits_out) {
+    if (n_t <= 256) {
+        *ts_out = 256;
+        *n_splits_out = 1;
+        return;
+    }
+    int want = (512 + n_kv_heads - 1) / n_kv_heads;
+    if (want > kMaxSplits) want = kMaxSplits;
+    int ts = ((n_t + want - 1) / want + 63) / 64 * 64;
+    if (ts < 64) ts = 64;
+    *ts_out = ts;
+    *n_splits_out = (n_t + ts - 1) / ts;
+}
+
 // Enqueue one forward pass for the B tokens / positions already in m->dtok /
 // m->dpos.  max_pos is the largest position among them (sizes the attention
 // scratch).  With want_logits the classifier and the running argmax follow.
@@ -932,7 +984,10 @@ extern "C" int l2_model_classifier(l2_model *m, const float *x_host, float *y_ho
 // residual add behind; w1|w3 with the ffn rmsnorm in front and the SiLU gate
 // behind; w2 with the residual add behind.  Every producer writes its result
 // in the input order (g_index) of whoever reads it next.
+static int forward_enqueue_dense(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits);
+
 static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits) {
+    if (m->d.group_size == 0) return forward_enqueue_dense(m, s, B, max_pos, want_logits);
     const l2_dims &d = m->d;
     const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
     hipStream_t st = m->stream;
@@ -968,21 +1023,9 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
             a.part = m->attn_part;
             a.n_heads = d.n_heads, a.n_kv_heads = d.n_kv_heads;
             a.max_splits = kMaxSplits;
-            const int n_t = max_pos + 1;
-            if (n_t <= 256) {
-                a.ts = 256;
-                a.n_splits = 1;
-            } else {
-                // two blocks per CU where the context allows it, at least 64 timesteps each
-                int want = (512 + d.n_kv_heads - 1) / d.n_kv_heads;
-                if (want > kMaxSplits) want = kMaxSplits;
-                int ts = ((n_t + want - 1) / want + 63) / 64 * 64;
-                if (ts < 64) ts = 64;
-                a.ts = ts;
-                a.n_splits = (n_t + ts - 1) / ts;
-                if (a.n_splits > kMaxSplits)
-                    return l2_fail(L2_ERR_RANGE, "attention: position %d needs %d splits", max_pos, a.n_splits);
-            }
+            attn_split_policy(max_pos + 1, d.n_kv_heads, &a.ts, &a.n_splits);
+            if (a.n_splits > kMaxSplits)
+                return l2_fail(L2_ERR_RANGE, "attention: position %d needs %d splits", max_pos, a.n_splits);
             LAUNCH(K_ATTENTION, attention_decode_launch(a, st));
         } else {
             LAUNCH(K_ROPE_KV, rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
@@ -1027,6 +1070,63 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
         (void)hid;
     }
     if (want_logits) // final rmsnorm + classifier (:288-297, B == 1 only) + running argmax
+        LAUNCH(K_CLASSIFIER, dense_matvec_launch(m->logits, m->wcls, m->x, m->rms_final, m->rms_eps, dim,
+                                                 d.vocab_size, m->amax, st));
+    return L2_OK;
+}
+
+// The same schedule for the model without quantisation (TransformerWeights, src/model.rs:36-67):
+// every projection is a dense matvec with its rmsnorm in front (q, k, v, w1, w3), the SiLU gate behind
+// (w3) or the residual add behind (wo, w2).  No act-order, so nothing is scattered.
+static int forward_enqueue_dense(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits) {
+    const l2_dims &d = m->d;
+    const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
+    hipStream_t st = m->stream;
+    {
+        ScatterTargets t{};
+        LAUNCH(K_EMBED, embed_launch(m->x, m->tok_emb, m->dtok, dim, B, t, m->amax, st));
+    }
+    auto dense = [&](const DevQLinear &w, const float *x, const float *wn, float *y, const float *res,
+                     const float *gate) {
+        DenseArgs a{};
+        a.y = y, a.w = w.dense, a.x = x, a.wn = wn, a.eps = m->rms_eps, a.in = w.in, a.out = w.out, a.batch = B;
+        a.res = res, a.gate = gate;
+        return dense_launch(a, st);
+    };
+    for (int l = 0; l < L; l++) {
+        const float *att_n = m->rms_att + (size_t)l * dim, *ffn_n = m->rms_ffn + (size_t)l * dim;
+        LAUNCH(K_Q4_QKV, dense(m->q[L2_WQ][l], m->x, att_n, m->qv, nullptr, nullptr)); // :217-226
+        L2_TRY(dense(m->q[L2_WK][l], m->x, att_n, m->kv, nullptr, nullptr));
+        L2_TRY(dense(m->q[L2_WV][l], m->x, att_n, m->vv, nullptr, nullptr));
+        float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
+        float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
+        if (B == 1) {
+            AttnDecode a{};
+            a.q = m->qv, a.k_new = m->kv, a.v_new = m->vv;
+            a.kcache = kc, a.vcache = vc;
+            a.cos_t = m->rope_cos, a.sin_t = m->rope_sin;
+            a.pos = max_pos;
+            a.out = m->attg, a.scatter = nullptr;
+            a.part = m->attn_part;
+            a.n_heads = d.n_heads, a.n_kv_heads = d.n_kv_heads;
+            a.max_splits = kMaxSplits;
+            attn_split_policy(max_pos + 1, d.n_kv_heads, &a.ts, &a.n_splits);
+            if (a.n_splits > kMaxSplits)
+                return l2_fail(L2_ERR_RANGE, "attention: position %d needs %d splits", max_pos, a.n_splits);
+            LAUNCH(K_ATTENTION, attention_decode_launch(a, st));
+        } else {
+            LAUNCH(K_ROPE_KV, rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
+                                             d.n_kv_heads, m->head_size, B, st));
+            LAUNCH(K_ATTENTION, attention_launch(m->attg, nullptr, m->qv, kc, vc, m->dpos, nullptr, d.n_heads,
+                                                 d.n_kv_heads, m->head_size, max_pos, B, st));
+        }
+        LAUNCH(K_Q4_WO, dense(m->q[L2_WO][l], m->attg, nullptr, m->x, m->x, nullptr));       // :260-264
+        LAUNCH(K_Q4_W13, dense(m->q[L2_W1][l], m->x, ffn_n, m->hd, nullptr, nullptr));        // :266-271
+        L2_TRY(dense(m->q[L2_W3][l], m->x, ffn_n, m->hg, nullptr, m->hd));                    // :272-276
+        LAUNCH(K_Q4_W2, dense(m->q[L2_W2][l], m->hg, nullptr, m->x, m->x, nullptr));          // :279-285
+        (void)hid;
+    }
+    if (want_logits)
         LAUNCH(K_CLASSIFIER, dense_matvec_launch(m->logits, m->wcls, m->x, m->rms_final, m->rms_eps, dim,
                                                  d.vocab_size, m->amax, st));
     return L2_OK;

@@ -136,113 +136,121 @@ __device__ __forceinline__ unsigned long long amax_key(float v, int idx) {
     return ((unsigned long long)u << 32) | (uint32_t)idx;
 }
 
-// Linear::matvec (src/model.rs:22-31) for the classifier: one wave per row,
-// x staged in LDS.  With wn set, x is first normalised as rmsnorm does
-// (src/models.rs:53-66, :288-295): the block stages wn[i]*x[i] and scales each
-// logit by ss = 1/sqrt(mean(x^2) + eps).  Optionally folds each logit into a
-// 64-bit (value,index) maximum, one atomic per wave.
+// Linear::matvec (src/model.rs:22-31): the classifier of every model and every
+// projection of the model without quantisation.  One wave per row, x staged in
+// LDS.  With wn set, x is first normalised as rmsnorm does (src/models.rs:53-66):
+// the block stages wn[i]*x[i] and scales each output by ss = 1/sqrt(mean(x^2) +
+// eps).  Epilogue, all optional: the SiLU gate out = silu(gate[o]) * out
+// (src/models.rs:92-98, gate = the w1 output when this is w3), the residual
+// add out = res[o] + out (:47-51), and the fold of (value, index) into a 64-bit
+// maximum, one atomic per wave.  blockIdx.y is the batch column.
 //
 // A wave takes R rows at a time and issues all R * KI loads of 16 bytes per
 // lane (32 in all) before the first FMA, every load unconditional: columns past
 // the end re-read the row's last 16 bytes against a zero of x, rows past the
-// end re-read the last row.
-template <int KI> // float4 per lane and row
-__global__ __launch_bounds__(256) void dense_matvec_kernel(float *y, const float *w, const float *x,
-                                                            const float *wn, float eps, int in, int out,
-                                                            unsigned long long *amax) {
+// end re-read the last row.  Inputs longer than 32 * 64 float4 take several
+// such passes over a row (R = 1) into the same accumulator.
+template <int KI> // float4 per lane, row and pass
+__global__ __launch_bounds__(256) void dense_matvec_kernel(const DenseArgs A) {
     constexpr int R = 32 / KI >= 1 ? 32 / KI : 1;
-    extern __shared__ float xs[]; // KI * 64 float4, zero beyond in
+    extern __shared__ float xs[]; // n_pass * KI * 64 float4, zero beyond in
     __shared__ float red[16];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: row addresses stay scalar
+    const int in = A.in, out = A.out;
     const int n4 = in >> 2;
-    const float4 *__restrict__ w4 = reinterpret_cast<const float4 *>(w);
+    const int n_pass = A.n_pass;
+    const int padded = n_pass * KI * 64;
+    const size_t bcol = blockIdx.y;
+    const float *__restrict__ x = A.x + bcol * in;
+    const float *__restrict__ wn = A.wn;
+    const float4 *__restrict__ w4 = reinterpret_cast<const float4 *>(A.w);
     const float4 *__restrict__ xs4 = reinterpret_cast<const float4 *>(xs);
 
-    constexpr int XL = (KI * 64 + 255) / 256;
-    float4 xv[XL], gv[XL];
-#pragma unroll
-    for (int r = 0; r < XL; r++) {
-        const int i = min(tid + r * 256, n4 - 1);
-        xv[r] = reinterpret_cast<const float4 *>(x)[i];
-        gv[r] = wn ? reinterpret_cast<const float4 *>(wn)[i] : make_float4(1.f, 1.f, 1.f, 1.f);
+    float ssq = 0.f;
+    for (int base = 0; base < padded; base += 256) {
+        const int i = base + tid;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < n4) {
+            v = reinterpret_cast<const float4 *>(x)[i];
+            if (wn) {
+                const float4 g = reinterpret_cast<const float4 *>(wn)[i];
+                ssq = fmaf(v.x, v.x, ssq);
+                ssq = fmaf(v.y, v.y, ssq);
+                ssq = fmaf(v.z, v.z, ssq);
+                ssq = fmaf(v.w, v.w, ssq);
+                v.x *= g.x;
+                v.y *= g.y;
+                v.z *= g.z;
+                v.w *= g.w;
+            }
+        }
+        if (i < padded) reinterpret_cast<float4 *>(xs)[i] = v;
     }
+    float ss = 1.0f;
+    if (wn) {
+        ssq = block_sum(ssq, red);
+        ssq /= (float)in;
+        ssq += A.eps;
+        ss = 1.0f / sqrtf(ssq);
+    }
+    __syncthreads();
 
     const int waves_total = gridDim.x * 4;
     const int o_first = (blockIdx.x * 4 + wave) * R;
-    uint32_t col[KI]; // byte offsets within a row
-#pragma unroll
-    for (int i = 0; i < KI; i++) col[i] = (uint32_t)min(i * 64 + lane, n4 - 1) << 4;
     float4 wv[R][KI];
-    auto load_tile = [&](int o) {
+    auto load_tile = [&](int o, int pass) {
 #pragma unroll
         for (int k = 0; k < R; k++) {
             // 32-bit byte offsets from the one base (the launcher checks that the matrix stays below 4 GiB)
             const uint32_t row = (uint32_t)min(o + k, out - 1) * ((uint32_t)n4 << 4);
 #pragma unroll
-            for (int i = 0; i < KI; i++)
-                wv[k][i] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(w4) + (row + col[i]));
+            for (int i = 0; i < KI; i++) {
+                const uint32_t col = (uint32_t)min((pass * KI + i) * 64 + lane, n4 - 1) << 4;
+                wv[k][i] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(w4) + (row + col));
+            }
         }
     };
-    float ss = 1.0f;
     unsigned long long key = 0ull;
-    auto finish_tile = [&](int o) {
+    float *__restrict__ y = A.y + bcol * out;
+    const float *__restrict__ res = A.res ? A.res + bcol * out : nullptr;
+    const float *__restrict__ gate = A.gate ? A.gate + bcol * out : nullptr;
+    for (int o = o_first; o < out; o += waves_total * R) {
         float a[R];
 #pragma unroll
         for (int k = 0; k < R; k++) a[k] = 0.f;
+        for (int pass = 0; pass < n_pass; pass++) {
+            __builtin_amdgcn_sched_barrier(0); // a pass's loads stay behind the pass before it: one set of registers
+            load_tile(o, pass);
+            __builtin_amdgcn_sched_barrier(0); // every load of the pass before its first FMA
 #pragma unroll
-        for (int i = 0; i < KI; i++) {
-            const float4 xx = xs4[i * 64 + lane];
+            for (int i = 0; i < KI; i++) {
+                const float4 xx = xs4[(pass * KI + i) * 64 + lane];
 #pragma unroll
-            for (int k = 0; k < R; k++) {
-                a[k] = fmaf(wv[k][i].x, xx.x, a[k]);
-                a[k] = fmaf(wv[k][i].y, xx.y, a[k]);
-                a[k] = fmaf(wv[k][i].z, xx.z, a[k]);
-                a[k] = fmaf(wv[k][i].w, xx.w, a[k]);
+                for (int k = 0; k < R; k++) {
+                    a[k] = fmaf(wv[k][i].x, xx.x, a[k]);
+                    a[k] = fmaf(wv[k][i].y, xx.y, a[k]);
+                    a[k] = fmaf(wv[k][i].z, xx.z, a[k]);
+                    a[k] = fmaf(wv[k][i].w, xx.w, a[k]);
+                }
             }
         }
 #pragma unroll
         for (int k = 0; k < R; k++) {
-            const float v = wave_sum(a[k]) * ss;
+            float v = wave_sum(a[k]) * ss;
             if (lane == 0 && o + k < out) {
+                if (gate) {
+                    const float g = gate[o + k];
+                    v = (g * (1.0f / (1.0f + expf(-g)))) * v;
+                }
+                if (res) v = res[o + k] + v;
                 y[o + k] = v;
                 const unsigned long long kk = amax_key(v, o + k);
                 key = kk > key ? kk : key;
             }
         }
-    };
-    float ssq = 0.f;
-#pragma unroll
-    for (int r = 0; r < XL; r++) {
-        const int i = tid + r * 256;
-        float4 v = xv[r];
-        if (i >= n4) v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (wn) {
-            ssq = fmaf(v.x, v.x, ssq);
-            ssq = fmaf(v.y, v.y, ssq);
-            ssq = fmaf(v.z, v.z, ssq);
-            ssq = fmaf(v.w, v.w, ssq);
-            v.x *= gv[r].x;
-            v.y *= gv[r].y;
-            v.z *= gv[r].z;
-            v.w *= gv[r].w;
-        }
-        if (i < KI * 64) reinterpret_cast<float4 *>(xs)[i] = v;
     }
-    if (wn) {
-        ssq = block_sum(ssq, red);
-        ssq /= (float)in;
-        ssq += eps;
-        ss = 1.0f / sqrtf(ssq);
-    }
-    __syncthreads();
-    for (int o = o_first; o < out; o += waves_total * R) {
-        __builtin_amdgcn_sched_barrier(0); // a tile's loads stay behind the tile before it: one set of registers
-        load_tile(o);
-        __builtin_amdgcn_sched_barrier(0); // every load of the tile before its first FMA
-        finish_tile(o);
-    }
-    if (lane == 0 && amax && key) atomicMax(amax, key);
+    if (lane == 0 && A.amax && key) atomicMax(A.amax, key);
 }
 
 // Greedy hand-over (src/inference.rs:154-162, 185-189): next is the forced
@@ -301,28 +309,46 @@ int rope_kv_launch(float *q, const float *k, const float *v, const int32_t *pos,
     return L2_OK;
 }
 
-int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
-                        unsigned long long *amax_key, hipStream_t st) {
-    if (in < 4 || in % 4 || in > 8192 || out < 1 || (size_t)in * out * 4 >= ((size_t)1 << 32))
-        return l2_fail(L2_ERR_ARG, "dense matvec: in=%d out=%d", in, out);
-    const int ki = (in / 4 + 63) / 64; // float4 per lane and row
+int dense_launch(const DenseArgs &a0, hipStream_t st) {
+    DenseArgs a = a0;
+    if (a.in < 4 || a.in % 4 || a.in > 32768 || a.out < 1 || a.batch < 1 ||
+        (size_t)a.in * a.out * 4 >= ((size_t)1 << 32))
+        return l2_fail(L2_ERR_ARG, "dense matvec: in=%d out=%d batch=%d", a.in, a.out, a.batch);
+    if (a.amax && a.batch != 1) return l2_fail(L2_ERR_ARG, "dense matvec: the running maximum takes one column");
+    const int ki = (a.in / 4 + 63) / 64; // float4 per lane and row
     const int KI = ki <= 4 ? 4 : ki <= 8 ? 8 : ki <= 16 ? 16 : ki <= 20 ? 20 : 32;
     const int R = 32 / KI >= 1 ? 32 / KI : 1;
+    a.n_pass = (ki + KI - 1) / KI;
     // three blocks per CU (the registers allow three waves per SIMD), fewer when the rows run out
-    int blocks = 3 * 256;
-    const int need = (out + 4 * R - 1) / (4 * R);
+    int blocks = (3 * 256 + a.batch - 1) / a.batch;
+    const int need = (a.out + 4 * R - 1) / (4 * R);
     if (blocks > need) blocks = need;
-    const size_t lds = (size_t)KI * 64 * 16;
-    dim3 grid(blocks), block(256);
+    const size_t lds = (size_t)a.n_pass * KI * 64 * 16;
+    dim3 grid(blocks, a.batch), block(256);
+    if (lds > 48 * 1024) {
+        static size_t raised = 0;
+        if (lds > raised) {
+            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(dense_matvec_kernel<32>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            raised = lds;
+        }
+    }
     switch (KI) {
-        case 4: hipLaunchKernelGGL(dense_matvec_kernel<4>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
-        case 8: hipLaunchKernelGGL(dense_matvec_kernel<8>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
-        case 16: hipLaunchKernelGGL(dense_matvec_kernel<16>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
-        case 20: hipLaunchKernelGGL(dense_matvec_kernel<20>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
-        default: hipLaunchKernelGGL(dense_matvec_kernel<32>, grid, block, lds, st, y, w, x, wn, eps, in, out, amax_key); break;
+        case 4: hipLaunchKernelGGL(dense_matvec_kernel<4>, grid, block, lds, st, a); break;
+        case 8: hipLaunchKernelGGL(dense_matvec_kernel<8>, grid, block, lds, st, a); break;
+        case 16: hipLaunchKernelGGL(dense_matvec_kernel<16>, grid, block, lds, st, a); break;
+        case 20: hipLaunchKernelGGL(dense_matvec_kernel<20>, grid, block, lds, st, a); break;
+        default: hipLaunchKernelGGL(dense_matvec_kernel<32>, grid, block, lds, st, a); break;
     }
     L2_HIP(hipGetLastError());
     return L2_OK;
+}
+
+int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
+                        unsigned long long *amax_key, hipStream_t st) {
+    DenseArgs a{};
+    a.y = y, a.w = w, a.x = x, a.wn = wn, a.eps = eps, a.in = in, a.out = out, a.amax = amax_key, a.batch = 1;
+    return dense_launch(a, st);
 }
 
 int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,

@@ -41,6 +41,7 @@ struct DevQLinear {
     const int32_t *g_index = nullptr; // [in]
     const int32_t *inv_index = nullptr; // [in], inv_index[g_index[j]] = j
     int in = 0, out = 0, groups = 0, group_size = 0;
+    const float *dense = nullptr;     // the model without quantisation: Linear<IN,OUT>.w [out][in]; the rest null
 };
 
 // ---- q4 matvec launch description ------------------------------------------
@@ -172,6 +173,20 @@ int attention_decode_launch(const AttnDecode &a, hipStream_t st);
 // wn == nullptr: plain Linear::matvec of x.
 int dense_matvec_launch(float *y, const float *w, const float *x, const float *wn, float eps, int in, int out,
                         unsigned long long *amax_key, hipStream_t st);
+// The general form: y[b] = epilogue(w (rmsnorm?)(x[b])) for `batch` columns (see dense_matvec_kernel).
+struct DenseArgs {
+    float *y;            // [batch][out]
+    const float *w;      // [out][in]
+    const float *x;      // [batch][in]
+    const float *wn;     // [in] or null: rmsnorm weight applied to x, with eps
+    float eps;
+    int in, out, batch;
+    unsigned long long *amax; // null, or the running (value, index) maximum (batch == 1)
+    const float *res;    // null, or [batch][out] added to the result (may alias y)
+    const float *gate;   // null, or [batch][out]: result = silu(gate) * result
+    int n_pass;          // set by the launcher
+};
+int dense_launch(const DenseArgs &a, hipStream_t st);
 // pos = dpos[0]; next = pos < n_prompt ? prompt[pos] : index(amax_key);
 // out_ids[pos - pos0] = next; tok[0] = next; dpos[0] = pos + 1.
 int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,

@@ -71,12 +71,16 @@ def groups_of(n_in: int, group_size: int) -> int:
 
 
 def qlinear_bytes(n_in: int, n_out: int, group_size: int) -> int:
+    if group_size == 0:  # the build without quantisation: a dense Linear<IN,OUT> (src/model.rs:11-15)
+        return n_out * n_in * 4
     g = groups_of(n_in, group_size)
     return n_out * (n_in // 8) * 4 + (n_out // 8) * g * 4 + n_out * g * 4 + n_in * 4
 
 
 def weights_bytes(d: Dims) -> int:
-    """size_of::<QTransformerWeights>() — what src/lib.rs:97 asserts the mmap length equals."""
+    """size_of::<QTransformerWeights>() — what src/lib.rs:97 asserts the mmap length equals.
+    group_size 0 (GROUPSIZE of the build without quantisation, src/constants.rs:58-61) gives
+    size_of::<TransformerWeights>() (src/model.rs:36-67): the same fields, every projection dense."""
     L, G = d.n_layers, d.group_size
     n = 4 + d.vocab_size * d.dim * 4 + L * d.dim * 4
     n += L * (2 * qlinear_bytes(d.dim, d.dim, G) + 2 * qlinear_bytes(d.dim, d.kv_dim, G))
@@ -194,6 +198,9 @@ def synth_weights_image(d: Dims, seed: int = 0, act_order: bool = True,
 
     def qlin_block(n_in, n_out):
         for _ in range(d.n_layers):
+            if d.group_size == 0:  # dense Linear, about the scale a trained projection has
+                f32(rng.normal(0.0, 1.0 / np.sqrt(n_in), size=(n_out, n_in)))
+                continue
             qw, qz, sc, gi = synth_qlinear(rng, n_in, n_out, d.group_size, act_order)
             i32(qw), i32(qz), f32(sc), i32(gi)
 

@@ -35,13 +35,15 @@ def _preset_for(path: str) -> ck.Dims:
     for name, base in ck.PRESETS.items():
         if size and name != size:
             continue
-        for g in ([group] if group else [128, 64, 32]):
+        # with features named and no `quantized` among them the build is the dense one (build.rs:16-38)
+        dense_only = bool(names) and "quantized" not in names and group is None
+        for g in ([0] if dense_only else [group] if group else [128, 64, 32, 0]):
             d = ck.preset(name, g)
             if (d.dim, d.hidden_dim, d.n_layers, d.n_heads) == (hdr["dim"], hdr["hidden_dim"], hdr["n_layers"],
                                                                 hdr["n_heads"]) and ck.checkpoint_bytes(d) == nbytes:
                 candidates.append(d)
     if not candidates:
-        raise ValueError(f"{path}: header {hdr} and size {nbytes} match no 7B/13B/70B x group_32/64/128 preset"
+        raise ValueError(f"{path}: header {hdr} and size {nbytes} match no 7B/13B/70B preset (group_32/64/128 or without quantisation)"
                          + (f" allowed by LLAMA2_RS_FEATURES={feats}" if feats else ""))
     return candidates[0]
 

@@ -62,6 +62,7 @@ typedef struct {
     const float *scales;    /* [OUT][GROUPS] */
     const int32_t *g_index; /* [IN] */
     int32_t in, out, groups;
+    const float *dense;     /* quant = "no": Linear<IN,OUT>.w [OUT][IN] (src/model.rs:11-15), the others null */
 } or_qlinear;
 
 typedef struct {
@@ -304,8 +305,23 @@ static size_t qlinear_bytes(int in, int out, int g) {
            (size_t)out * groups * 4 + (size_t)in * 4;
 }
 
+/* size_of::<TransformerWeights>() (src/model.rs:36-67): the build without quantisation,
+ * GROUPSIZE = 0 (src/constants.rs:58-61); every projection a dense Linear. */
+static size_t dense_weights_bytes(const or_dims *d) {
+    const int hs = d->dim / d->n_heads;
+    const size_t kv_dim = (size_t)d->n_kv_heads * hs, dim = (size_t)d->dim, hid = (size_t)d->hidden_dim;
+    const size_t L = (size_t)d->n_layers;
+    size_t n = 4 + (size_t)d->vocab_size * dim * 4 + L * dim * 4;
+    n += L * (dim * dim + 2 * kv_dim * dim + dim * dim) * 4; /* wq wk wv wo */
+    n += L * dim * 4;
+    n += L * 3 * hid * dim * 4;                              /* w1 w2 w3 */
+    n += dim * 4 + (size_t)d->seq_len * (hs / 2) * 4 * 2 + (size_t)d->vocab_size * dim * 4;
+    return n;
+}
+
 /* size_of::<QTransformerWeights>() for these dims (the part after the 28-byte header). */
 size_t or_weights_bytes(const or_dims *d) {
+    if (d->group_size == 0) return dense_weights_bytes(d);
     const int hs = d->dim / d->n_heads;
     const int kv_dim = d->n_kv_heads * hs;
     const size_t L = (size_t)d->n_layers;
@@ -325,6 +341,15 @@ size_t or_weights_bytes(const or_dims *d) {
 }
 
 static const char *take_qlinears(const char *p, or_qlinear *ql, int L, int in, int out, int g) {
+    if (g == 0) { /* dense Linear<IN,OUT> */
+        for (int l = 0; l < L; l++) {
+            ql[l].in = in;
+            ql[l].out = out;
+            ql[l].dense = (const float *)p;
+            p += (size_t)out * in * 4;
+        }
+        return p;
+    }
     const int groups = (int)div_up(in, g);
     for (int l = 0; l < L; l++) {
         ql[l].in = in;
@@ -416,6 +441,10 @@ float *or_state_key_cache(or_state *s) { return s->key_cache; }
 float *or_state_value_cache(or_state *s) { return s->value_cache; }
 
 static void qmv(const or_qlinear *q, int g, int B, const float *x, float *y) {
+    if (q->dense) {
+        or_dense_matvec(q->dense, q->in, q->out, B, x, y);
+        return;
+    }
     or_qmatvec(q->qweight, q->qzeros, q->scales, q->g_index, q->in, q->out, g, B, x, y);
 }
 

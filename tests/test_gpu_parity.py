@@ -168,6 +168,54 @@ def test_decode_attention_long_context(ops, oracle, n_heads, n_kv, ctx):
     o.close()
 
 
+DENSE = ck.Dims(dim=512, hidden_dim=640, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=260,
+                seq_len=80, group_size=0)
+DENSE_WIDE = ck.Dims(dim=256, hidden_dim=9216, n_layers=1, n_heads=2, n_kv_heads=2, vocab_size=64,
+                     seq_len=32, group_size=0)   # w2 takes two passes over a row (in > 8192)
+
+
+@pytest.mark.parametrize("dims", [DENSE, DENSE_WIDE], ids=["gqa", "long_rows"])
+def test_model_without_quantisation(ops, oracle, dims, tmp_path):
+    """group_size 0 = the reference's build without the `quantized` feature: TransformerWeights
+    (src/model.rs:36-67), every projection a dense Linear; same loop, same oracle."""
+    img = ck.synth_weights_image(dims, seed=5)
+    path = str(tmp_path / "dense.bin")
+    ck.write_checkpoint(path, dims, img)
+    m = ops.Model(path, dims)
+    o = oracle.Model(img, dims)
+    o.new_state()
+    toks = [1, 5, 60, 17, 3]
+    for pos, t in enumerate(toks):
+        want = o.transformer([t], [pos])
+        got = m.forward([t], [pos])
+        assert nrel(got, want) < REL_FP32, pos
+        assert int(np.argmax(got)) == oracle.argmax(want)
+    # a chunk of 4 continues the sequence; then the greedy loop with the prefill ladder
+    nxt, poss = [7, 8, 9, 10], list(range(len(toks), len(toks) + 4))
+    assert m.forward(nxt, poss) is None
+    o.transformer(nxt, poss)
+    ko, vo = o.kv_cache()
+    k, v = m.read_kv(dims.n_layers - 1, 0, len(toks) + 4)
+    assert nrel(k, ko[-1, :len(toks) + 4]) < REL_FP32
+    assert nrel(v, vo[-1, :len(toks) + 4]) < REL_FP32
+    prompt = np.array([3, 9, 33, 12, 50, 7, 21], np.int32)
+    got, _ = m.generate_greedy(prompt, 20, use_prefill=True)
+    want = o.generate_greedy(prompt, 20, use_prefill=True)
+    np.testing.assert_array_equal(got, want)
+    # the operator entry point is Linear::matvec<B>
+    from llama2_rs import _lib
+    import tests.test_oracle_loop as tol
+    W = tol._split_image(img, dims)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((3, dims.hidden_dim)).astype(np.float32)
+    assert nrel(m.qmatvec(0, _lib.W2, x), (W["w2"][0] @ x.astype(np.float64).T).T) < REL_FP32
+    from llama2_rs._lib import L2Error
+    with pytest.raises(L2Error):
+        m.set_prefill_mode(1)   # the MFMA prefill path is the quantised model's
+    m.close()
+    o.close()
+
+
 def test_kv_snapshot_restore(ops):
     """read_kv / write_kv: a cache restored into a fresh state continues with the same tokens."""
     dims = TINY_GQA

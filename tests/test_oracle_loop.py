@@ -25,8 +25,11 @@ def _split_image(img, d):
 
     def qlin(n_in, n_out):
         out = []
-        g = ck.groups_of(n_in, d.group_size)
+        g = ck.groups_of(n_in, d.group_size) if d.group_size else 0
         for _ in range(d.n_layers):
+            if d.group_size == 0:  # dense Linear (src/model.rs:11-15)
+                out.append(take(n_out * n_in, np.float32).reshape(n_out, n_in).astype(np.float64))
+                continue
             qw = take(n_out * n_in // 8, np.int32).reshape(n_out, n_in // 8)
             qz = take(n_out // 8 * g, np.int32).reshape(n_out // 8, g)
             sc = take(n_out * g, np.float32).reshape(n_out, g)
@@ -91,7 +94,11 @@ def _forward_fp64(w, d, tokens):
     return logits
 
 
-@pytest.mark.parametrize("dims", [TINY, TINY_GQA], ids=["mha_g64", "gqa_g128"])
+DENSE_GQA = ck.Dims(dim=512, hidden_dim=640, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=260,
+                    seq_len=80, group_size=0)  # the build without quantisation (GROUPSIZE 0)
+
+
+@pytest.mark.parametrize("dims", [TINY, TINY_GQA, DENSE_GQA], ids=["mha_g64", "gqa_g128", "dense_gqa"])
 def test_transformer_against_fp64_numpy(oracle, dims):
     img = ck.synth_weights_image(dims, seed=11)
     m = oracle.Model(img, dims)
@@ -121,6 +128,11 @@ def test_struct_sizes_of_the_three_presets():
     assert round(ck.checkpoint_bytes(ck.preset("70B", 64)) / 1e9, 3) == 41.167
     # one q_proj of the 7B preset: the byte count quoted for the standalone matvec
     assert ck.qlinear_bytes(4096, 4096, 128) == 8_388_608 + 65_536 + 524_288 + 16_384
+    # size_of::<TransformerWeights>() of the 7B build without quantisation (src/model.rs:36-67), by hand:
+    # eps + 2 tables of 32000x4096 + 32 layers of (2 norms + 4 x 4096^2 + 3 x 4096x11008) + final norm + freq tables
+    dense = 4 + 2 * 32000 * 4096 * 4 + 32 * (2 * 4096 + 4 * 4096 * 4096 + 3 * 4096 * 11008) * 4 + 4096 * 4 \
+        + 2 * 2048 * 64 * 4
+    assert ck.weights_bytes(ck.preset("7B", 0)) == dense
 
 
 @pytest.mark.parametrize("n_prompt", [0, 1, 2, 3, 7, 23, 70])
