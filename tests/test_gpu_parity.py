@@ -62,6 +62,42 @@ def test_qmatvec_vs_oracle(ops, oracle, n_in, n_out, G, B):
     q.close()
 
 
+_ALT_FORM_SNIPPET = r"""
+import sys, numpy as np
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[2])
+from llama2_rs import ops, checkpoint as ck
+from oracle import oracle_lib as o
+worst = 0.0
+for n_in, n_out, G, B in ((4096, 512, 128, 1), (1024, 264, 64, 3), (11008, 256, 128, 1), (512, 40, 32, 2)):
+    rng = np.random.default_rng(n_in + n_out)
+    qw, qz, sc, gi = ck.synth_qlinear(rng, n_in, n_out, G)
+    x = rng.standard_normal((B, n_in)).astype(np.float32)
+    want = np.asarray(o.qmatvec(qw, qz, sc, gi, G, x), np.float64)
+    q = ops.QLinear(qw, qz, sc, gi, G)
+    got = np.asarray(q.matvec(x), np.float64)
+    scale = np.maximum(np.abs(want), np.sqrt(np.mean(want ** 2)) + 1e-30)
+    worst = max(worst, float(np.max(np.abs(got - want) / scale)))
+    q.close()
+print("WORST", worst)
+"""
+
+
+@pytest.mark.parametrize("form", ["tile", "idot"])
+def test_selectable_kernel_forms(form):
+    """L2_Q4_IMPL=tile|idot select other forms of the q4 kernel when the library is loaded; each runs
+    the same parity check in a process of its own."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, L2_Q4_IMPL=form)
+    r = subprocess.run([sys.executable, "-c", _ALT_FORM_SNIPPET, os.path.join(root, "llama2.rs_amd"), root],
+                       capture_output=True, text=True, env=env, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    worst = float(r.stdout.strip().split("WORST")[-1])
+    assert worst < REL_FP32, (form, worst)
+
+
 def test_qmatvec_unit_vectors_and_linearity(ops):
     rng = np.random.default_rng(5)
     n_in, n_out, G = 512, 96, 64
