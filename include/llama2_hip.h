@@ -125,6 +125,12 @@ int l2_prefill_supported(const l2_model *m);
 /* Choose how B > 1 is computed (L2_PREFILL_*).  Default L2_PREFILL_FP32. */
 int l2_model_set_prefill_mode(l2_model *m, int mode);
 
+/* Decode steps (B = 1 inside l2_generate_greedy, l2_decode_greedy, l2_decode_bench) as captured HIP graphs,
+ * one per bucket of positions [0,256), [256,512), [512,1024), ..., replayed with one host call per token.
+ * No counterpart in the reference.  Off by default (the step is bound by its kernels, not by their
+ * launches); on, the results are the same tokens.  Environment: L2_STEP_GRAPH=1 turns it on at load. */
+int l2_model_set_step_graph(l2_model *m, int on);
+
 /* RunState::new (src/models.rs:36-41): zero-filled fp32 KV cache
  * [n_layers][max_seq][n_kv_heads][head_size] x2 in device memory. */
 int l2_state_new(l2_model *m, l2_state **out);

@@ -4,6 +4,7 @@
 // (src/inference.rs:16-193), driving the HIP kernels.  Nothing here computes on
 // the CPU except the one-time RoPE angle table and the synthetic-image
 // generator.
+#include <map>
 #include <fcntl.h>
 #include <math.h>
 #include <stdarg.h>
@@ -299,6 +300,14 @@ struct l2_model {
     unsigned long long *amax = nullptr;
     int32_t *dprompt = nullptr, *dout_ids = nullptr;
     int cap_prompt = 0, cap_out = 0;
+    // The decode step as a HIP graph (one per bucket of positions, kept in the state).  Off by default: a
+    // replayed step takes the host out of the loop (one call per token instead of some 160), but the step is
+    // bound by its kernels, not by their launches, and reading the position from device memory costs the
+    // attention kernel a little (7B: 625 tok/s replayed, 629 launched).
+    int32_t *dloop = nullptr;     // device {n_prompt, pos0} of the running loop, read by the captured next_token launch
+    uint64_t buf_epoch = 1;       // bumped whenever a buffer a captured step points at is reallocated
+    bool capturing = false;       // forward_enqueue: take the position from m->dpos, size attention for max_pos
+    bool use_graph = false;
     // scratch for the operator-level entry points
     float *op_x = nullptr, *op_xg = nullptr, *op_y = nullptr;
     size_t op_cap = 0;
@@ -340,11 +349,20 @@ static constexpr int kMaxSplits = 64;
         }                                                                           \
     } while (0)
 
+struct StepGraph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    uint64_t epoch = 0;
+};
+
 struct l2_state {
     l2_model *m = nullptr;
     float *kcache = nullptr, *vcache = nullptr; // [L][max_seq][kv_dim]
     size_t elems = 0;
+    std::map<int, StepGraph> steps; // captured decode step per upper bound of the position
 };
+
+static void step_graph_drop(StepGraph &g);
 
 struct l2_qlinear {
     DevQLinear q;
@@ -416,6 +434,7 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
     L2_TRY(require_device());
 
     l2_model *m = new l2_model();
+    m->use_graph = getenv("L2_STEP_GRAPH") != nullptr; // also l2_model_set_step_graph
     m->d = *dims;
     m->max_seq = max_seq;
     m->head_size = dims->dim / dims->n_heads;
@@ -620,7 +639,7 @@ extern "C" void l2_model_close(l2_model *m) {
     if (!m) return;
     if (m->stream) (void)hipStreamSynchronize(m->stream);
     void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->dwn, m->attn_part, m->x, m->xq, m->xk,
-                    m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->hd, m->logits, m->dtok, m->dpos,
+                    m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->hd, m->logits, m->dtok, m->dpos, m->dloop,
                     m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y, m->h16a, m->h16b, m->h16c,
                     m->hb, m->hb2, m->ssb, m->gemm_ws};
     for (void *p : ptrs) dfree(p);
@@ -644,6 +663,12 @@ extern "C" int l2_model_max_seq(const l2_model *m) { return m ? m->max_seq : 0; 
 
 extern "C" int l2_prefill_supported(const l2_model *m) { return m ? 1 : 0; }
 
+extern "C" int l2_model_set_step_graph(l2_model *m, int on) {
+    if (!m) return l2_fail(L2_ERR_ARG, "null model");
+    m->use_graph = on != 0;
+    return L2_OK;
+}
+
 extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
     if (!m) return l2_fail(L2_ERR_ARG, "null model");
     if (mode != L2_PREFILL_FP32 && mode != L2_PREFILL_MFMA) return l2_fail(L2_ERR_ARG, "prefill mode %d", mode);
@@ -661,6 +686,7 @@ static int ensure_batch_mfma(l2_model *m, int B);
 static int ensure_batch(l2_model *m, int B) {
     if (B <= m->cap_B) return L2_OK;
     L2_HIP(hipStreamSynchronize(m->stream));
+    m->buf_epoch++;
     float **bufs[] = {&m->x, &m->xq, &m->xk, &m->xv, &m->qv, &m->kv, &m->vv, &m->attg, &m->x1, &m->x3, &m->hg};
     for (float **b : bufs) {
         dfree(*b);
@@ -690,6 +716,7 @@ static int ensure_batch(l2_model *m, int B) {
     L2_TRY(dalloc(&m->dtok, (size_t)B));
     L2_TRY(dalloc(&m->dpos, (size_t)B));
     if (!m->logits) L2_TRY(dalloc(&m->logits, (size_t)m->d.vocab_size));
+    if (!m->dloop) L2_TRY(dalloc(&m->dloop, (size_t)2));
     m->cap_B = B;
     return L2_OK;
 }
@@ -720,6 +747,7 @@ extern "C" int l2_state_new(l2_model *m, l2_state **out) {
 extern "C" void l2_state_free(l2_state *s) {
     if (!s) return;
     if (s->m && s->m->stream) (void)hipStreamSynchronize(s->m->stream);
+    for (auto &kv : s->steps) step_graph_drop(kv.second);
     dfree(s->kcache);
     dfree(s->vcache);
     delete s;
@@ -1019,6 +1047,7 @@ static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool wa
             a.kcache = kc, a.vcache = vc;
             a.cos_t = m->rope_cos, a.sin_t = m->rope_sin;
             a.pos = max_pos;
+            a.dpos = m->capturing ? m->dpos : nullptr; // a captured step serves every position up to max_pos
             a.out = m->attg, a.scatter = wo.inv_index;
             a.part = m->attn_part;
             a.n_heads = d.n_heads, a.n_kv_heads = d.n_kv_heads;
@@ -1106,6 +1135,7 @@ static int forward_enqueue_dense(l2_model *m, l2_state *s, int B, int max_pos, b
             a.kcache = kc, a.vcache = vc;
             a.cos_t = m->rope_cos, a.sin_t = m->rope_sin;
             a.pos = max_pos;
+            a.dpos = m->capturing ? m->dpos : nullptr; // a captured step serves every position up to max_pos
             a.out = m->attg, a.scatter = nullptr;
             a.part = m->attn_part;
             a.n_heads = d.n_heads, a.n_kv_heads = d.n_kv_heads;
@@ -1285,15 +1315,20 @@ extern "C" int l2_forward(l2_model *m, l2_state *s, const int32_t *tokens, const
     return L2_OK;
 }
 
+static int ensure_loop_buffers(l2_model *m, int n_prompt, int n_out);
+static int loop_begin(l2_model *m, int n_prompt, int pos0);
+static int loop_step(l2_model *m, l2_state *s, int pos, int n_prompt, int pos0);
+
 extern "C" int l2_decode_greedy(l2_model *m, l2_state *s, int32_t token, int32_t pos, int32_t *next) {
     if (!m || !s || !next) return l2_fail(L2_ERR_ARG, "null argument");
     if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
     int max_pos = 0;
     L2_TRY(check_tokens(m, &token, &pos, 1, &max_pos));
     L2_TRY(ensure_batch(m, 1));
-    L2_HIP(hipMemcpyAsync(m->dtok, &token, 4, hipMemcpyHostToDevice, m->stream));
-    L2_HIP(hipMemcpyAsync(m->dpos, &pos, 4, hipMemcpyHostToDevice, m->stream));
-    L2_TRY(forward_enqueue(m, s, 1, pos, true));
+    L2_TRY(ensure_loop_buffers(m, 1, 1));
+    L2_TRY(set_i32_launch(m->dtok, token, m->dpos, pos, m->stream));
+    L2_TRY(loop_begin(m, 0, pos));
+    L2_TRY(loop_step(m, s, pos, 0, pos)); // the argmax stays in m->amax; the hand-over it also does is harmless
     unsigned long long key = 0;
     L2_HIP(hipMemcpyAsync(&key, m->amax, 8, hipMemcpyDeviceToHost, m->stream));
     L2_HIP(hipStreamSynchronize(m->stream));
@@ -1304,6 +1339,7 @@ extern "C" int l2_decode_greedy(l2_model *m, l2_state *s, int32_t token, int32_t
 static int ensure_loop_buffers(l2_model *m, int n_prompt, int n_out) {
     if (n_prompt > m->cap_prompt) {
         L2_HIP(hipStreamSynchronize(m->stream));
+        m->buf_epoch++;
         dfree(m->dprompt);
         m->dprompt = nullptr;
         m->cap_prompt = 0;
@@ -1312,6 +1348,7 @@ static int ensure_loop_buffers(l2_model *m, int n_prompt, int n_out) {
     }
     if (n_out > m->cap_out) {
         L2_HIP(hipStreamSynchronize(m->stream));
+        m->buf_epoch++;
         dfree(m->dout_ids);
         m->dout_ids = nullptr;
         m->cap_out = 0;
@@ -1326,10 +1363,71 @@ static int ensure_loop_buffers(l2_model *m, int n_prompt, int n_out) {
 // then next = prompt[pos] if still inside the prompt else argmax
 // (src/inference.rs:146-162), stored to out_ids[pos - pos0], fed back as the
 // token, and the device position advanced.
-static int loop_step(l2_model *m, l2_state *s, int pos, int n_prompt, int pos0) {
+static int loop_step_eager(l2_model *m, l2_state *s, int pos, int n_prompt, int pos0) {
     L2_TRY(forward_enqueue(m, s, 1, pos, true));
     LAUNCH(K_NEXT_TOKEN, next_token_launch(m->amax, m->dprompt, n_prompt, m->dpos, m->dout_ids, pos0, m->dtok, m->stream));
     return L2_OK;
+}
+
+static void step_graph_drop(StepGraph &g) {
+    if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    if (g.graph) (void)hipGraphDestroy(g.graph);
+    g = StepGraph{};
+}
+
+// The captured form of the same step for every position below `upper`: the kernels read the position, the
+// prompt length and the first position of the loop from device memory (m->dpos, m->dloop), attention is
+// cut for `upper` timesteps and blocks beyond the current position leave at once.
+static int step_graph_get(l2_model *m, l2_state *s, int upper, hipGraphExec_t *out) {
+    StepGraph &g = s->steps[upper];
+    if (g.exec && g.epoch == m->buf_epoch) {
+        *out = g.exec;
+        return L2_OK;
+    }
+    step_graph_drop(g);
+    L2_HIP(hipStreamBeginCapture(m->stream, hipStreamCaptureModeRelaxed));
+    m->capturing = true;
+    int rc = forward_enqueue(m, s, 1, upper - 1, true);
+    if (rc == L2_OK)
+        rc = next_token_launch(m->amax, m->dprompt, 0, m->dpos, m->dout_ids, 0, m->dtok, m->stream, m->dloop);
+    m->capturing = false;
+    hipGraph_t graph = nullptr;
+    const hipError_t e = hipStreamEndCapture(m->stream, &graph);
+    if (rc != L2_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (e != hipSuccess) return l2_fail(L2_ERR_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    g.graph = graph;
+    const hipError_t e2 = hipGraphInstantiate(&g.exec, graph, nullptr, nullptr, 0);
+    if (e2 != hipSuccess) {
+        step_graph_drop(g);
+        return l2_fail(L2_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e2));
+    }
+    g.epoch = m->buf_epoch;
+    *out = g.exec;
+    return L2_OK;
+}
+
+// Positions are served in buckets [0, 256), [256, 512), [512, 1024), ...: one captured step each.
+static int step_bucket(const l2_model *m, int pos) {
+    long upper = 256;
+    while (upper <= pos) upper *= 2;
+    if (upper > m->max_seq) upper = m->max_seq;
+    return (int)upper;
+}
+
+// One step of a loop whose {n_prompt, pos0} are already in m->dloop (loop_begin).
+static int loop_step(l2_model *m, l2_state *s, int pos, int n_prompt, int pos0) {
+    if (!m->use_graph || m->prof_on) return loop_step_eager(m, s, pos, n_prompt, pos0);
+    hipGraphExec_t exec = nullptr;
+    L2_TRY(step_graph_get(m, s, step_bucket(m, pos), &exec));
+    L2_HIP(hipGraphLaunch(exec, m->stream));
+    return L2_OK;
+}
+
+static int loop_begin(l2_model *m, int n_prompt, int pos0) {
+    return set_i32_launch(m->dloop, n_prompt, m->dloop + 1, pos0, m->stream);
 }
 
 extern "C" int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *prompt, int n_prompt, int steps,
@@ -1372,6 +1470,7 @@ extern "C" int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *promp
     const int32_t first = pos == 0 ? 1 : prompt[pos - 1]; // :128-132
     L2_TRY(set_i32_launch(m->dtok, first, m->dpos, pos, m->stream));
     const int pos0 = pos;
+    L2_TRY(loop_begin(m, n_prompt, pos0));
     int n = 0;
     while (pos < steps) { // :141
         L2_TRY(loop_step(m, s, pos, n_prompt, pos0));
@@ -1424,6 +1523,14 @@ extern "C" int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t 
     L2_TRY(ensure_batch(m, 1));
     L2_TRY(ensure_loop_buffers(m, 1, n_tokens));
     L2_TRY(set_i32_launch(m->dtok, token, m->dpos, pos, m->stream));
+    L2_TRY(loop_begin(m, 0, pos));
+    if (m->use_graph) { // capture (if need be) outside the timed region
+        hipGraphExec_t exec = nullptr;
+        for (int b = step_bucket(m, pos);; b = step_bucket(m, b)) {
+            L2_TRY(step_graph_get(m, s, b, &exec));
+            if (b > pos + n_tokens - 1 || b >= m->max_seq) break;
+        }
+    }
     hipEvent_t e0, e1;
     L2_HIP(hipEventCreate(&e0));
     L2_HIP(hipEventCreate(&e1));
@@ -1452,6 +1559,7 @@ extern "C" int l2_decode_profile(l2_model *m, l2_state *s, int32_t token, int32_
     L2_TRY(ensure_batch(m, 1));
     L2_TRY(ensure_loop_buffers(m, 1, n_tokens));
     L2_TRY(set_i32_launch(m->dtok, token, m->dpos, pos, m->stream));
+    L2_TRY(loop_begin(m, 0, pos));
     L2_HIP(hipStreamSynchronize(m->stream));
     m->prof.clear();
     m->prof_on = true;

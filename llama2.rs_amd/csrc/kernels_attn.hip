@@ -68,7 +68,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
     __shared__ float kvnew[2][HS];
     __shared__ float comb[NWV][QG][HS + 2];
     const int kvh = blockIdx.x, sp = blockIdx.y;
-    const int pos = A.pos;
+    const int pos = A.dpos ? A.dpos[0] : A.pos;
     const int t0 = sp * A.ts;
     if (t0 > pos) return;
     const int t1 = min(t0 + A.ts, pos + 1);
@@ -483,7 +483,7 @@ __global__ __launch_bounds__(512) void attn_combine_kernel(const AttnDecode A) {
     __shared__ float den_s;
     __shared__ float red[3][HS];
     const int h = blockIdx.x, tid = threadIdx.x, d = tid & 127, grp = tid >> 7;
-    const int pos = A.pos;
+    const int pos = A.dpos ? A.dpos[0] : A.pos;
     const int ns = min(A.n_splits, pos / A.ts + 1);
     const float *p = A.part + (size_t)h * A.max_splits * (HS + 2);
     if (tid < 64) {

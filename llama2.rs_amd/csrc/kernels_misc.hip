@@ -257,8 +257,13 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(const DenseArgs A) {
 // prompt token while pos < n_prompt, else the argmax; it is recorded, fed back
 // as the next input token, and the position advances -- all without the host.
 __global__ void next_token_kernel(const unsigned long long *amax, const int32_t *prompt, int n_prompt,
-                                  int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok) {
+                                  int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok,
+                                  const int32_t *loop_params) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
+        if (loop_params) {
+            n_prompt = loop_params[0];
+            pos0 = loop_params[1];
+        }
         const int pos = dpos[0];
         const int32_t next = pos < n_prompt ? prompt[pos] : (int32_t)(amax[0] & 0xFFFFFFFFull);
         if (out_ids) out_ids[pos - pos0] = next;
@@ -352,9 +357,10 @@ int dense_matvec_launch(float *y, const float *w, const float *x, const float *w
 }
 
 int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,
-                      int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok, hipStream_t st) {
+                      int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok, hipStream_t st,
+                      const int32_t *loop_params) {
     hipLaunchKernelGGL(next_token_kernel, dim3(1), dim3(64), 0, st, amax_key, prompt, n_prompt, dpos,
-                       out_ids, pos0, tok);
+                       out_ids, pos0, tok, loop_params);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }

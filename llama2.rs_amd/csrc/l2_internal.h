@@ -159,6 +159,7 @@ struct AttnDecode {
     float *kcache, *vcache;          // this layer: [max_seq][kv_dim]
     const float *cos_t, *sin_t;      // [max_seq][head_size/2]
     int pos;                         // position of this step (the host knows it; no device read in front of the loads)
+    const int32_t *dpos;             // if set, the position is read from here instead (a captured step serves many positions)
     float *out;                      // [dim], written through scatter
     const int32_t *scatter;
     float *part;                     // split workspace: [n_heads][max_splits][130]
@@ -189,8 +190,10 @@ struct DenseArgs {
 int dense_launch(const DenseArgs &a, hipStream_t st);
 // pos = dpos[0]; next = pos < n_prompt ? prompt[pos] : index(amax_key);
 // out_ids[pos - pos0] = next; tok[0] = next; dpos[0] = pos + 1.
+// With loop_params (device: {n_prompt, pos0}) those two come from there, so that one captured launch serves any loop.
 int next_token_launch(const unsigned long long *amax_key, const int32_t *prompt, int n_prompt,
-                      int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok, hipStream_t st);
+                      int32_t *dpos, int32_t *out_ids, int pos0, int32_t *tok, hipStream_t st,
+                      const int32_t *loop_params = nullptr);
 // p[0] = a; if (q) q[0] = b.  Scalars travel as kernel arguments, never as
 // asynchronous copies from the caller's stack.
 int set_i32_launch(int32_t *p, int32_t a, int32_t *q, int32_t b, hipStream_t st);

@@ -56,6 +56,7 @@ SIGNATURES = {
     "l2_model_max_seq": (_I, [_VP]),
     "l2_prefill_supported": (_I, [_VP]),
     "l2_model_set_prefill_mode": (_I, [_VP, _I]),
+    "l2_model_set_step_graph": (_I, [_VP, _I]),
     "l2_state_new": (_I, [_VP, C.POINTER(_VP)]),
     "l2_state_free": (None, [_VP]),
     "l2_state_reset": (_I, [_VP]),

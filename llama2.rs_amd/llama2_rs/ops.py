@@ -146,6 +146,10 @@ class Model:
         """_lib.PREFILL_FP32 (default, identical to B=1) or _lib.PREFILL_MFMA (fp16 tiles, 2e-3)."""
         check(lib().l2_model_set_prefill_mode(self.h, mode))
 
+    def set_step_graph(self, on: bool):
+        """Replay decode steps as captured HIP graphs (off by default)."""
+        check(lib().l2_model_set_step_graph(self.h, 1 if on else 0))
+
     def qmatvec(self, layer: int, proj: int, x) -> np.ndarray:
         x = _f32(x)
         one = x.ndim == 1

@@ -252,6 +252,37 @@ def test_model_without_quantisation(ops, oracle, dims, tmp_path):
     o.close()
 
 
+@pytest.mark.parametrize("dims", [TINY_GQA, DENSE], ids=["q4_gqa", "dense"])
+def test_decode_steps_as_graphs(ops, oracle, dims):
+    """Captured decode steps give the tokens of the launched ones: replays are interleaved with eager
+    forward passes, host synchronisation, a reset and a second loop with another prompt length."""
+    img = ck.synth_weights_image(dims, seed=4)
+    m = ops.Model(img, dims)
+    o = oracle.Model(img, dims)
+    m.set_step_graph(True)
+    for n_prompt, steps in ((6, 30), (0, 12), (17, 40)):
+        prompt = np.random.default_rng(n_prompt).integers(0, dims.vocab_size, size=n_prompt).astype(np.int32)
+        got, _ = m.generate_greedy(prompt, steps, use_prefill=False)
+        want = o.generate_greedy(prompt, steps, use_prefill=False)
+        np.testing.assert_array_equal(got, want)
+        # eager work between loops: a forward pass with logits, then single replayed steps
+        m.reset()
+        o.new_state()
+        logits = m.forward([1], [0])
+        assert nrel(logits, o.transformer([1], [0])) < REL_FP32
+        tok = 1
+        for pos in range(5):
+            nxt = m.decode_greedy(tok, pos)
+            ref = oracle.argmax(o.transformer([tok], [pos]))
+            assert nxt == ref, pos
+            tok = nxt
+    m.set_step_graph(False)
+    got2, _ = m.generate_greedy(prompt, steps, use_prefill=True)
+    np.testing.assert_array_equal(got2, o.generate_greedy(prompt, steps, use_prefill=True))
+    m.close()
+    o.close()
+
+
 def test_kv_snapshot_restore(ops):
     """read_kv / write_kv: a cache restored into a fresh state continues with the same tokens."""
     dims = TINY_GQA
