@@ -333,7 +333,11 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     }
 
     const int n_rows = row1 - row0;
-    const int n_tiles = (n_rows + TR - 1) / TR;
+    // Steps of the longest stream; whole tiles of P steps run in the loop, what is left runs once after it,
+    // straight-line and without refills, so that the loop body stays one block (and its waits exact).
+    const int n_steps = (n_rows + S - 1) / S;
+    const int n_full = n_steps / P;
+    const int n_rem = n_steps - n_full * P;
     int buf = 0;
     // Enter the loop with no load outstanding (the primed rows arrived while x
     // was staged). The compiler's wait counts inside the loop are then those of
@@ -358,7 +362,58 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
 #pragma unroll
     for (int t = 0; t < 3; t++) idx_p[t] = t < n_scatter ? sc_idx[t] : reinterpret_cast<const int32_t *>(sc[0]);
 
-    for (int tile = 0; tile < n_tiles; tile++) {
+    // one row (row pair) of this stream: dequantised dot product of the lane's chunk -> pr
+    auto row_dot = [&](int o, const RowData(&d)[NM], float(&pr)[NM]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            const int zn = (d[q].z >> (4 * (o & 7))) & 15;
+            if constexpr (IDOT) {
+                const float f = chunk_idot(d[q].w, xp[q]);
+                pr[q] = (d[q].s * xdelta[q]) * fmaf(-(float)(zn - 7), sx[q], f);
+            } else {
+                const float p = chunk_dot(d[q].w, x[q]);
+                const float z1 = (float)(zn + 1);
+                pr[q] = d[q].s * fmaf(p, 512.0f, -z1 * sx[q]);
+            }
+        }
+    };
+    // 64 partials -> 4 (one per 16-lane row) -> the tile's slot for this row
+    auto row_fold = [&](int u, const float(&pr)[NM]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            float v = pr[q];
+            v += dpp_xchg<0xB1>(v);
+            v += dpp_xchg<0x4E>(v);
+            v += dpp_xchg<0x141>(v);
+            v += dpp_xchg<0x140>(v);
+            if ((lane & 15) == 0) part[buf][u * S + stream][q][kslice * 4 + (lane >> 4)] = v;
+        }
+    };
+    // one thread per row of the tile: fixed-order sum of the partials, then the epilogue
+    auto tile_finish = [&](int eo, float res_v, const uint32_t(&sidx)[3]) __attribute__((always_inline)) {
+        float sum[NM];
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            float a = 0.f;
+#pragma unroll
+            for (int k = 0; k < PW; k++) a += part[buf][tid][q][k];
+            sum[q] = a;
+        }
+        float v = sum[0] * ss;
+        if (PAIR) { // silu(w1 x) * (w3 x), src/models.rs:92-98
+            const float u2 = sum[NM - 1] * ss;
+            v = v * (1.0f / (1.0f + expf(-v)));
+            v = v * u2;
+        } else if (epi_kind == Q4_EPI_RESIDUAL) {
+            v = res_v + v;
+        }
+        if (epi_kind != Q4_EPI_SCATTER_ONLY) yout[out_base + eo] = v;
+#pragma unroll
+        for (int t = 0; t < 3; t++)
+            if (t < n_scatter) st_at(sc_out[t], ((uint32_t)out_base + sidx[t]) << 2, v); // 32-bit offset: nothing widens the loaded index
+    };
+
+    for (int tile = 0; tile < n_full; tile++) {
         // The lanes that finish this tile's rows fetch what the epilogue reads
         // (residual, scatter indices) now: by the time it is needed, P rows of
         // younger loads stand behind it and the wait leaves those in flight.
@@ -374,20 +429,8 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
 #pragma unroll
         for (int u = 0; u < P; u++) {
             const int i = tile * P + u;
-            const int o = row0 + stream + i * S;
             float pr[NM];
-#pragma unroll
-            for (int q = 0; q < NM; q++) {
-                const int zn = (pipe[u][q].z >> (4 * (o & 7))) & 15;
-                if constexpr (IDOT) {
-                    const float f = chunk_idot(pipe[u][q].w, xp[q]);
-                    pr[q] = (pipe[u][q].s * xdelta[q]) * fmaf(-(float)(zn - 7), sx[q], f);
-                } else {
-                    const float p = chunk_dot(pipe[u][q].w, x[q]);
-                    const float z1 = (float)(zn + 1);
-                    pr[q] = pipe[u][q].s * fmaf(p, 512.0f, -z1 * sx[q]);
-                }
-            }
+            row_dot(row0 + stream + i * S, pipe[u], pr);
             // Refill this slot with row i + P, after its last use and not before:
             // a load hoisted above the row's arithmetic makes the compiler copy
             // live registers of the other slots, and each copy waits on its load.
@@ -398,42 +441,35 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
             __builtin_amdgcn_sched_barrier(0);
             fetch(i + P, pipe[u]);
             __builtin_amdgcn_sched_barrier(0);
+            row_fold(u, pr);
+        }
+        __syncthreads();
+        if (epi) tile_finish(eo, res_v, sidx);
+        buf ^= 1;
+        Q4S_STAMP(4);
+    }
+    if (n_rem > 0) { // the rows already in the pipe: no refill, nothing younger to leave in flight
+        const int eo = row0 + n_full * TR + tid;
+        const bool epi = tid < TR && eo < row1;
+        float res_v = 0.f;
+        uint32_t sidx[3] = {0, 0, 0};
+        if (epi) {
+            res_v = res_p[eo];
 #pragma unroll
-            for (int q = 0; q < NM; q++) {
-                float v = pr[q];
-                v += dpp_xchg<0xB1>(v);
-                v += dpp_xchg<0x4E>(v);
-                v += dpp_xchg<0x141>(v);
-                v += dpp_xchg<0x140>(v);
-                if ((lane & 15) == 0) part[buf][u * S + stream][q][kslice * 4 + (lane >> 4)] = v;
+            for (int t = 0; t < 3; t++) sidx[t] = (uint32_t)idx_p[t][eo];
+        }
+#pragma unroll
+        for (int u = 0; u < P - 1; u++) {
+            if (u < n_rem) {
+                float pr[NM];
+                row_dot(row0 + stream + (n_full * P + u) * S, pipe[u], pr);
+                row_fold(u, pr);
             }
         }
         __syncthreads();
-        if (epi) {
-            float sum[NM];
-#pragma unroll
-            for (int q = 0; q < NM; q++) {
-                float a = 0.f;
-#pragma unroll
-                for (int k = 0; k < PW; k++) a += part[buf][tid][q][k];
-                sum[q] = a;
-            }
-            float v = sum[0] * ss;
-            if (PAIR) { // silu(w1 x) * (w3 x), src/models.rs:92-98
-                const float u2 = sum[NM - 1] * ss;
-                v = v * (1.0f / (1.0f + expf(-v)));
-                v = v * u2;
-            } else if (epi_kind == Q4_EPI_RESIDUAL) {
-                v = res_v + v;
-            }
-            if (epi_kind != Q4_EPI_SCATTER_ONLY) yout[out_base + eo] = v;
-#pragma unroll
-            for (int t = 0; t < 3; t++)
-                if (t < n_scatter) st_at(sc_out[t], ((uint32_t)out_base + sidx[t]) << 2, v); // 32-bit offset: nothing widens the loaded index
-        }
-        buf ^= 1;
-        Q4S_STAMP(4 + (tile + 1 == n_tiles));
+        if (epi) tile_finish(eo, res_v, sidx);
     }
+    Q4S_STAMP(5);
 }
 
 #if defined(Q4S_TS)
