@@ -118,7 +118,8 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps = the prompt, forced through the loop (default 16; 32 for 13B, as its config asks)")
     ap.add_argument("--model", default="7B", choices=["7B", "13B", "70B"])
     ap.add_argument("--group", type=int, default=0, help="group size (default: 128, 64 for 70B)")
     ap.add_argument("--kv-prefill", type=int, default=0,
@@ -135,6 +136,8 @@ def main() -> int:
         print("bench.py: this build runs on exactly one GPU (no sharding, no collectives); "
               f"--gpus {a.gpus} is not supported", file=sys.stderr)
         return 2
+    if a.warmup is None:
+        a.warmup = 32 if a.model == "13B" else 16
     K, W = a.steps, a.warmup
     if K < 1 or W < 0:
         print("bench.py: --steps must be >= 1 and --warmup >= 0", file=sys.stderr)

@@ -674,9 +674,11 @@ extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
     if (mode != L2_PREFILL_FP32 && mode != L2_PREFILL_MFMA) return l2_fail(L2_ERR_ARG, "prefill mode %d", mode);
     if (mode == L2_PREFILL_MFMA && m->d.group_size == 0)
         return l2_fail(L2_ERR_ARG, "the MFMA prefill path is the quantised model's");
-    if (mode == L2_PREFILL_MFMA && !(q4_gemm_supports(m->d.dim, m->d.dim) && q4_gemm_supports(m->d.hidden_dim, m->kv_dim) &&
-                                     q4_gemm_supports(m->d.dim, m->d.hidden_dim)))
-        return l2_fail(L2_ERR_ARG, "the MFMA prefill path needs dim and hidden_dim to be multiples of 64");
+    const int G = m->d.group_size;
+    if (mode == L2_PREFILL_MFMA && !(q4_gemm_supports(m->d.dim, m->d.dim, G) && q4_gemm_supports(m->d.hidden_dim, m->kv_dim, G) &&
+                                     q4_gemm_supports(m->d.dim, m->d.hidden_dim, G)))
+        return l2_fail(L2_ERR_ARG, "the MFMA prefill path needs dim and hidden_dim to be multiples of 128 (of 2 groups for "
+                                   "group sizes 64 and 128) and output sizes to be multiples of 32");
     m->prefill_mode = mode;
     return L2_OK;
 }
@@ -956,7 +958,7 @@ extern "C" int l2_model_qmatvec(l2_model *m, int layer, int proj, const float *x
         L2_HIP(hipStreamSynchronize(st));
         return L2_OK;
     }
-    if (B > 1 && m->prefill_mode == L2_PREFILL_MFMA && q4_gemm_supports(q.in, q.out)) {
+    if (B > 1 && m->prefill_mode == L2_PREFILL_MFMA && q4_gemm_supports(q.in, q.out, q.group_size)) {
         // the prefill form of the same operator: gather, round to fp16, dequant -> MFMA
         hipStream_t st = m->stream;
         L2_TRY(ensure_batch_mfma(m, B));

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     constexpr int TN = 32 * NB;
     constexpr bool SA = G >= 64; // scale after the group's partial sum
     extern __shared__ _Float16 xs[]; // [2][TN][kXRow]
-    __shared__ float gsc[2][128];    // fp32 scales of the block's 128 rows for the current group
+    __shared__ float gsc[2][kGemmPW][128]; // fp32 scales of the block's 128 rows, PW groups at a time
     const int in = L.in;
     const int n_k = in / KSTEP; // K iterations
 
@@ -139,7 +139,9 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
 
     const int o_lane = rb * 128 + wave * 32 + r;
     const int orow = min(o_lane, n_out - 1);
-    const int grow = min(rb * 128 + (tid & 127), n_out - 1); // the row whose group scale this thread fetches
+    // scale-after form: the thread fetches the scales of row `grow` for two of every PW groups
+    const int grow = min(rb * 128 + (tid & 127), n_out - 1);
+    const int ghalf = tid >> 7;
 
     f16v acc[NB];  // running result
     f16v accg[NB]; // partial sum of the current group (SA only)
@@ -154,15 +156,15 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     // this block's slice of K, in whole groups
     const int ks = blockIdx.z;
     const int n_grp = n_k / KPG;
-    const int kit0 = (int)((long)n_grp * ks / KS) * KPG;
-    const int kit1 = (int)((long)n_grp * (ks + 1) / KS) * KPG;
+    // slices start on an even group: the scales are fetched as aligned pairs
+    const int kit0 = ((int)((long)n_grp * ks / KS) & ~1) * KPG;
+    const int kit1 = ks + 1 == KS ? n_k : ((int)((long)n_grp * (ks + 1) / KS) & ~1) * KPG;
     const int n_it = kit1 - kit0;
 
     struct WStage {
         uint4 w[W];
         int32_t z;
         float s;  // this lane's row, scaled form only
-        float gs; // row `grow`, scale-after form only
     };
     const void *qw_base = M.qweight;
     const void *qz_base = M.qzeros;
@@ -174,13 +176,22 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
         for (int sw = 0; sw < W; sw++)
             d.w[sw] = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc * (2 * W) + 2 * sw + h) << 4);
         d.z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
-        if constexpr (SA) {
-            d.gs = ld_at<float>(sc_base, (uint32_t)(grow * groups + kc / KPG) << 2);
+        if constexpr (SA)
             d.s = 0.f;
-        } else {
+        else
             d.s = ld_at<float>(sc_base, (uint32_t)(orow * groups + g) << 2);
-            d.gs = 0.f;
-        }
+    };
+    // Scale-after form: one 8-byte load per thread and PW K steps (a K step is a group there) instead of
+    // one scattered 4-byte load per thread and step.  Block j of PW groups starts at group kit0 + PW * j;
+    // pairs past the row's last group re-read its last pair (their steps are never run).
+    static_assert(!SA || KPG == 1, "scale-after form: a K step is one group");
+    auto fetch_gs = [&](int j) {
+        const int ge = min(kit0 + PW * j + 2 * ghalf, groups - 2);
+        return ld_at<float2>(sc_base, (uint32_t)(grow * groups + ge) << 2);
+    };
+    auto store_gs = [&](int j, const float2 v) {
+        gsc[j & 1][2 * ghalf][tid & 127] = v.x;
+        gsc[j & 1][2 * ghalf + 1][tid & 127] = v.y;
     };
     // staging map: thread -> (token, 16-byte segment) x (TN*8/256) pieces
     constexpr int SEGS = KSTEP / 8; // 16-byte segments per token and K step
@@ -211,13 +222,15 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
 
     XStage xr[XP];
     WStage wr[PW];
+    float2 gs2 = make_float2(0.f, 0.f);
+    if constexpr (SA) gs2 = fetch_gs(0);
 #pragma unroll
     for (int j = 0; j < XP; j++) fetch_x(kit0 + j, xr[j]);
 #pragma unroll
     for (int j = 0; j < PW; j++) fetch_w(kit0 + j, wr[j]);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the loop's waits then reflect its own order only
     store_x(0, xr[0]);
-    if (SA && tid < 128) gsc[(kit0 / KPG) & 1][tid] = wr[0].gs;
+    if constexpr (SA) store_gs(0, gs2);
     __syncthreads();
     Q4G_STAMP(1);
 
@@ -247,6 +260,8 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             __builtin_amdgcn_sched_barrier(0);
             fetch_w(kit + PW, wr[u]);
             fetch_x(kit + XP, xr[u % XP]);
+            if constexpr (SA)
+                if (u == 0) gs2 = fetch_gs(base / PW + 1); // the next PW groups' scales
             __builtin_amdgcn_sched_barrier(0);
             const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
             // W * 4 steps of 16 k.  The operands of step i + 1 (two LDS reads per token tile, the
@@ -277,10 +292,10 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             }
             if (SA && (u + 1) % KPG == 0) {
                 // end of a group: fold its partial sum into the result with the fp32 scale of each row
-                const int gb = (kit / KPG) & 1;
+                const int gb = (base / PW) & 1;
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][wave * 32 + q * 8 + h * 4]);
+                    const float4 sv = *reinterpret_cast<const float4 *>(&gsc[gb][u][wave * 32 + q * 8 + h * 4]);
                     const float svv[4] = {sv.x, sv.y, sv.z, sv.w};
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++)
@@ -290,8 +305,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                             accg[nb][4 * q + e] = 0.f;
                         }
                 }
-                // the next group's scales (fetched PW - 1 steps ago with the next step's weights)
-                if (tid < 128) gsc[gb ^ 1][tid] = wr[(u + 1) % PW].gs;
+                if (u == PW - 1) store_gs(base / PW + 1, gs2); // fetched at the first step of this round
             }
             // the next step's activation tile was fetched XP - 1 steps ago
             store_x(buf ^ 1, xr[(u + 1) % XP]);
@@ -463,13 +477,13 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     const int NB = B > 32 ? 2 : 1;
     const int TN = 32 * NB;
     const int t_tiles = (B + TN - 1) / TN;
-    // K slices: aim at ~2 blocks per CU, whole groups per slice, at most 8
+    // K slices: as many as keep the grid within one round of 2 blocks per CU, whole groups per slice, at most 8
     // K step: 128 where a group is at least that long (half the block barriers per k), else 64
     constexpr int KSTEP = G >= 128 ? 128 : 64;
     const int n_grp = (L.in / KSTEP) / (G / KSTEP > 0 ? G / KSTEP : 1);
-    int KS = (512 + total * t_tiles - 1) / (total * t_tiles);
+    int KS = (2 * cu_count()) / (total * t_tiles); // all blocks resident at once: two per CU
     if (KS > 8) KS = 8;
-    if (KS > n_grp) KS = n_grp;
+    if (KS > n_grp / 2) KS = n_grp / 2; // slices start on even groups
     if (KS < 1) KS = 1;
     while (KS > 1 && (size_t)KS * B * rows > ws_floats) KS--;
     dim3 grid(total, t_tiles, KS), block(256);
@@ -494,6 +508,8 @@ int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, floa
                    hipStream_t st) {
     if (L.n_mats < 1 || L.n_mats > 3) return l2_fail(L2_ERR_ARG, "q4 gemm: n_mats=%d", L.n_mats);
     if (L.in % 128 != 0 || L.in % L.group_size != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d must be a multiple of 128", L.in);
+    if (L.group_size >= 64 && (L.in / L.group_size) % 2 != 0)
+        return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d is an odd number of groups of %d", L.in, L.group_size);
     for (int i = 0; i < L.n_mats; i++)
         if (L.m[i].out % 32 != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: out=%d must be a multiple of 32", L.m[i].out);
     if (L.pair) return l2_fail(L2_ERR_ARG, "q4 gemm: pair launches are not supported");
@@ -505,7 +521,11 @@ int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, floa
     return l2_fail(L2_ERR_ARG, "q4 gemm: group size %d", L.group_size);
 }
 
-bool q4_gemm_supports(int in, int out) { return in % 128 == 0 && out % 32 == 0; }
+bool q4_gemm_supports(int in, int out, int group_size) {
+    if (in % 128 != 0 || out % 32 != 0 || group_size <= 0 || in % group_size != 0) return false;
+    // groups of 64 and 128: the group scales are fetched as aligned pairs
+    return group_size < 64 || (in / group_size) % 2 == 0;
+}
 
 int prep_f16_multi_launch(const PrepList &P, int n, int B, hipStream_t st) {
     if (n % 8 || P.n_mats < 1 || P.n_mats > 3) return l2_fail(L2_ERR_ARG, "prep: n=%d, %d vectors", n, P.n_mats);

@@ -480,18 +480,6 @@ extern "C" int l2_debug_q4_ts(unsigned long long *out, int n) {
 namespace {
 #endif
 
-int cu_count() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
-    }
-    return n;
-}
-
 // Rows per block for a block of NW waves and tiles of TR rows: a whole number of rounds over the CUs, as
 // many blocks per CU as 16 waves and the LDS allow; every block gets the same number of rows; several
 // matrices round up separately and the grid stays within one round.

@@ -12,6 +12,19 @@
 
 #include "../../include/llama2_hip.h"
 
+// Compute units of the current device (256 on MI355X); asked once.
+inline int cu_count() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
 // ---- error plumbing -------------------------------------------------------
 int l2_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 
@@ -109,7 +122,7 @@ struct XhList {
 // Epilogues as in the matvec (no pair launches).  ws: workspace of ws_floats floats for split-K partial
 // tiles (the launcher uses as many K slices as fit).
 int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st);
-bool q4_gemm_supports(int in, int out);
+bool q4_gemm_supports(int in, int out, int group_size);
 // out_f16[b][j'] = fp16(x[b][j] * (wn ? wn[j] : 1)), j' = j with the order (0,4,1,5,2,6,3,7) inside every 8.
 int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st);
 // The same for up to three vectors of one length in one launch (q|k|v, w1|w3 inputs).
