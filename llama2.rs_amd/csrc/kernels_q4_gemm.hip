@@ -372,12 +372,13 @@ extern "C" int l2_debug_gemm_ts(unsigned long long *out, int n) {
 namespace {
 #endif
 
-// Adds the KS partial tiles of a split-K GEMM in slice order and runs the epilogue.
-// grid: (ceil(sum_out / 256), B); the matrices of the launch are laid end to end.
+// Adds the KS partial tiles of a split-K GEMM in slice order and runs the epilogue; a thread owns four
+// consecutive outputs of one token (every `out` is a multiple of 32).
+// grid: (ceil(sum_out / 1024), B); the matrices of the launch are laid end to end.
 __global__ __launch_bounds__(256) void q4_gemm_reduce_kernel(const Q4Launch L, const float *__restrict__ ss,
                                                              const float *__restrict__ ws, int KS) {
     const int t = blockIdx.y;
-    int o = blockIdx.x * 256 + threadIdx.x;
+    int o = (blockIdx.x * 256 + threadIdx.x) * 4;
     int mi = 0;
     size_t ws_base = 0;
     const int B = L.batch;
@@ -388,14 +389,31 @@ __global__ __launch_bounds__(256) void q4_gemm_reduce_kernel(const Q4Launch L, c
     }
     const Q4Mat &M = L.m[mi];
     if (o >= M.out) return;
-    float v = 0.f;
-    for (int ks = 0; ks < KS; ks++) v += ws[ws_base + ((size_t)ks * B + t) * M.out + o];
-    if (ss) v *= ss[t];
+    const float *p = ws + ws_base + (size_t)t * M.out + o;
+    const size_t slice = (size_t)B * M.out;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int ks = 0; ks < KS; ks++) {
+        const float4 a = *reinterpret_cast<const float4 *>(p + ks * slice);
+        v.x += a.x, v.y += a.y, v.z += a.z, v.w += a.w;
+    }
+    if (ss) {
+        const float sc = ss[t];
+        v.x *= sc, v.y *= sc, v.z *= sc, v.w *= sc;
+    }
     const Q4Epi &E = L.e;
     const size_t row = (size_t)t * M.out;
-    if (E.kind == Q4_EPI_RESIDUAL) v += E.res[row + o];
-    if (E.kind != Q4_EPI_SCATTER_ONLY) M.y[row + o] = v;
-    for (int c = 0; c < E.n_scatter; c++) E.sc_out[c][row + E.sc_idx[c][o]] = v;
+    if (E.kind == Q4_EPI_RESIDUAL) {
+        const float4 r = *reinterpret_cast<const float4 *>(E.res + row + o);
+        v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
+    }
+    if (E.kind != Q4_EPI_SCATTER_ONLY) *reinterpret_cast<float4 *>(M.y + row + o) = v;
+    const float vals[4] = {v.x, v.y, v.z, v.w};
+    for (int c = 0; c < E.n_scatter; c++) {
+        const int4 idx = *reinterpret_cast<const int4 *>(E.sc_idx[c] + o);
+        const int id[4] = {idx.x, idx.y, idx.z, idx.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) E.sc_out[c][row + id[e]] = vals[e];
+    }
 }
 
 // fp32 [B][n] (already in the consumer's g_index order) -> fp16 [B][n], times the
@@ -496,7 +514,7 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     }
     L2_HIP(hipGetLastError());
     if (KS > 1) {
-        hipLaunchKernelGGL(q4_gemm_reduce_kernel, dim3((unsigned)((rows + 255) / 256), B), dim3(256), 0, st, L, ss, ws, KS);
+        hipLaunchKernelGGL(q4_gemm_reduce_kernel, dim3((unsigned)((rows + 1023) / 1024), B), dim3(256), 0, st, L, ss, ws, KS);
         L2_HIP(hipGetLastError());
     }
     return L2_OK;
