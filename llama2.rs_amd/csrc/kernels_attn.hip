@@ -474,6 +474,214 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(float *__restrict__ o
     }
 }
 
+// Chunk attention on the matrix cores, all in fp32 (v_mfma_f32_32x32x2_f32), for the prefill mode that
+// hands fp16 activations to the next GEMM.  Same function as attn_prefill_kernel (src/models.rs:131-176,
+// causal per query over the cache rows 0..pos).
+//
+// A block of 8 waves owns 32 columns of one kv head: column n = (query ct*32/QG + n/QG, head kvh*QG + n%QG).
+// Wave w takes the key tiles w, w+8, ... of 32 cache rows each and keeps a running (m, l, O) of its own;
+// the block merges the eight at the end.  Per tile, with lane = (n = lane%32, h = lane/32):
+//   S^T = K Q^T      A: lane (key n, h) holds K[key][64h + s], B: lane (column n, h) holds Q[n][64h + s]
+//                    (the contraction index of MFMA step s and half h is d = 64h + s: each lane reads
+//                    256 contiguous bytes of its key row), 64 steps.
+//   C layout         lane (column n, h), register r -> key (r/4)*8 + 4h + r%4: a lane holds 16 scores of
+//                    ITS column, so the running maximum and sum are per-lane work plus one exchange
+//                    between the two halves.
+//   O^T += V^T P^T   step s, half h contracts over key (s/4)*8 + 4h + s%4, which is the lane's own
+//                    register s of P: the B operand needs no data movement.  A: lane (d-row n, h) reads
+//                    V[key][32*mt + n] from the wave's LDS tile; 4 tiles of 32 d, 16 steps each.
+template <int QG>
+__global__ __launch_bounds__(512) void attn_prefill_mfma_kernel(_Float16 *__restrict__ out_h, const float *__restrict__ q,
+                                                                 const float *__restrict__ kc, const float *__restrict__ vc,
+                                                                 const int32_t *__restrict__ pos,
+                                                                 const int32_t *__restrict__ scatter, int n_heads,
+                                                                 int n_kv_heads, int B, int max_pos) {
+    constexpr int HS = 128, NWV = 8, TK = 32, QPT = 32 / QG;
+    constexpr int kQRow = 33;      // floats per d-row of the transposed Q tile
+    constexpr int kVRow = HS + 4;  // floats per key row of a staged V tile
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    extern __shared__ float smem[];
+    float *qst = smem;                                  // [HS][kQRow]: Q^T of the block's 32 columns
+    __shared__ float m_s[NWV][32], l_s[NWV][32];
+    const int kvh = blockIdx.x, ct = blockIdx.y;
+    const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    float *vs = smem + HS * kQRow + wave * (TK * kVRow); // this wave's V tile, later its partial O^T [HS][32]
+
+    const float scale = 1.44269504088896340736f / sqrtf((float)HS);
+    const uint32_t row_bytes = (uint32_t)kv_dim * 4u;
+    const int last_row = max_pos; // the last cache row written: loads clamp to it and wait for nothing
+
+    // K: this lane's half of its key row; V: the tile row by row, 16 bytes per lane and load.  Rows past
+    // the end re-read the last row (masked below), so the loads are unconditional.
+    float4 kr[16], vr[16];
+    auto fetch_k = [&](int kt) {
+        const int tk = min(kt * TK + n, last_row);
+        const uint32_t off = __umul24(tk, row_bytes) + (uint32_t)(kvh * HS + 64 * h) * 4u;
+#pragma unroll
+        for (int i = 0; i < 16; i++) kr[i] = ld_at<float4>(kc, off + 16 * i);
+    };
+    auto fetch_v = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int f = i * 64 + lane;
+            const int tv = min(kt * TK + (f >> 5), last_row);
+            vr[i] = ld_at<float4>(vc, __umul24(tv, row_bytes) + (uint32_t)(kvh * HS + 4 * (f & 31)) * 4u);
+        }
+    };
+    fetch_k(wave);
+    fetch_v(wave);
+    __builtin_amdgcn_sched_barrier(0);
+    // positions of the 32 columns; the block's tiles end with the last row any of them sees
+    const int my_qi = ct * QPT + n / QG;
+    const int my_pos = my_qi < B ? pos[my_qi] : -1;
+    int t_end = my_pos + 1;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) t_end = max(t_end, __shfl_xor(t_end, off));
+    t_end = __builtin_amdgcn_readfirstlane(t_end);
+    const int n_kt = (t_end + TK - 1) / TK;
+
+    {   // Q^T of the 32 columns: all eight loads of a thread in flight, then the LDS writes
+        float qreg[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int idx = u * 512 + tid;
+            const int col = idx >> 7, d = idx & 127;
+            const int qi = min(ct * QPT + col / QG, B - 1);
+            qreg[u] = q[(size_t)qi * dim + (kvh * QG + col % QG) * HS + d];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int idx = u * 512 + tid;
+            qst[(idx & 127) * kQRow + (idx >> 7)] = qreg[u];
+        }
+    }
+    __syncthreads();
+
+    float m = kNoScore, l = 0.f;
+    v16f o[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[mt][r] = 0.f;
+
+    for (int kt = wave; kt < n_kt; kt += NWV) {
+        const int t0 = kt * TK;
+        v16f sacc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+        // the Q operands of steps 4i+4..4i+7 are read from LDS while the MFMAs of steps 4i..4i+3 run
+        float qv[2][4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) qv[0][e] = qst[(64 * h + e) * kQRow + n];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float kk[4] = {kr[i].x, kr[i].y, kr[i].z, kr[i].w};
+            if (i + 1 < 16) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) qv[(i + 1) & 1][e] = qst[(64 * h + 4 * (i + 1) + e) * kQRow + n];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 4; e++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[e], qv[i & 1][e], sacc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        fetch_k(kt + NWV); // the next tile's keys travel while this tile's softmax and P V run
+        __builtin_amdgcn_sched_barrier(0);
+        // the V tile into the wave's own LDS region (the wave's LDS accesses execute in order)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int f = i * 64 + lane;
+            *reinterpret_cast<float4 *>(&vs[(f >> 5) * kVRow + 4 * (f & 31)]) = vr[i];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_v(kt + NWV);
+        __builtin_amdgcn_sched_barrier(0);
+        // scores of this lane's column, running maximum shared by the two halves of the column
+        float sc[16];
+        float mx = m;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int key = t0 + (r >> 2) * 8 + 4 * h + (r & 3);
+            sc[r] = key <= my_pos ? sacc[r] * scale : kNoScore;
+            mx = fmaxf(mx, sc[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        if (__any(mx > m)) {
+            const float c = exp2_fast(m - mx);
+            l *= c;
+#pragma unroll
+            for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[mt][r] *= c;
+            m = mx;
+        }
+        float pr[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int key = t0 + (r >> 2) * 8 + 4 * h + (r & 3);
+            pr[r] = key <= my_pos ? exp2_fast(sc[r] - m) : 0.f;
+            l += pr[r];
+        }
+        // likewise the V operands: those of step st + 1 are read while the four MFMAs of step st run
+        float vv[2][4];
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) vv[0][mt] = vs[(4 * h) * kVRow + 32 * mt + n];
+#pragma unroll
+        for (int st = 0; st < 16; st++) {
+            if (st + 1 < 16) {
+                const int key = ((st + 1) >> 2) * 8 + 4 * h + ((st + 1) & 3);
+#pragma unroll
+                for (int mt = 0; mt < 4; mt++) vv[(st + 1) & 1][mt] = vs[key * kVRow + 32 * mt + n];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int mt = 0; mt < 4; mt++)
+                o[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[st & 1][mt], pr[st], o[mt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // this wave's (m, l, O^T) -> LDS; O^T [d][column] over the wave's V region
+    l += __shfl_xor(l, 32);
+    if (h == 0) {
+        m_s[wave][n] = m;
+        l_s[wave][n] = l;
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) vs[(32 * mt + (r >> 2) * 8 + 4 * h + (r & 3)) * 32 + n] = o[mt][r];
+    __syncthreads();
+    const float *part = smem + HS * kQRow;
+    // a thread's column is the same in all eight passes; its scatter targets are fetched together
+    const int col = tid & 31;
+    const int qi = ct * QPT + col / QG;
+    int dst[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        const int i = (kvh * QG + col % QG) * HS + u * 16 + (tid >> 5);
+        dst[u] = scatter ? scatter[i] : i;
+    }
+    if (qi >= B) return;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        const int d = u * 16 + (tid >> 5);
+        float M = m_s[0][col];
+#pragma unroll
+        for (int w = 1; w < NWV; w++) M = fmaxf(M, m_s[w][col]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWV; w++) {
+            const float e = exp2_fast(m_s[w][col] - M);
+            num = fmaf(e, part[w * (TK * kVRow) + d * 32 + col], num);
+            den = fmaf(e, l_s[w][col], den);
+        }
+        out_h[(size_t)qi * dim + h16_slot(dst[u])] = (_Float16)(num / den); // the order the next GEMM reads
+    }
+}
+
 // Merge the splits of one q head: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s.
 // Wave 0 turns the (m_s, l_s) of up to 64 splits into weights; 4 groups of 128
 // threads then sum the weighted partial outputs, every load independent.
@@ -541,11 +749,34 @@ int attention_decode_launch(const AttnDecode &a, hipStream_t st) {
 int attention_launch(float *out, void *out_f16, const float *q, const float *kcache_l, const float *vcache_l,
                      const int32_t *pos, const int32_t *scatter, int n_heads, int n_kv_heads,
                      int head_size, int max_pos, int B, hipStream_t st) {
-    (void)max_pos;
     if (head_size != 128) return l2_fail(L2_ERR_ARG, "attention: head_size=%d (128 only)", head_size);
     const int qg = n_heads / n_kv_heads;
     if (qg != 1 && qg != 2 && qg != 4 && qg != 8)
         return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
+    if (out_f16) { // the matrix-core form: 32 columns (queries x heads of the group) per block
+        constexpr size_t lds = (size_t)(128 * 33 + 8 * 32 * 132) * sizeof(float);
+        dim3 grid(n_kv_heads, (B * qg + 31) / 32), block(512);
+        auto launch = [&](auto kern) {
+            static bool raised = false; // per instantiation
+            if (!raised) {
+                if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)lds) != hipSuccess)
+                    return l2_fail(L2_ERR_HIP, "attention: %zu bytes of LDS refused", lds);
+                raised = true;
+            }
+            hipLaunchKernelGGL(kern, grid, block, lds, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads,
+                               n_kv_heads, B, max_pos);
+            return (int)L2_OK;
+        };
+        switch (qg) {
+            case 1: L2_TRY(launch(attn_prefill_mfma_kernel<1>)); break;
+            case 2: L2_TRY(launch(attn_prefill_mfma_kernel<2>)); break;
+            case 4: L2_TRY(launch(attn_prefill_mfma_kernel<4>)); break;
+            default: L2_TRY(launch(attn_prefill_mfma_kernel<8>)); break;
+        }
+        L2_HIP(hipGetLastError());
+        return L2_OK;
+    }
     const int qpb = 8 / qg;
     dim3 grid(n_kv_heads, (B + qpb - 1) / qpb), block(256);
     switch (qg) {
