@@ -432,6 +432,42 @@ def test_text_generate_api(ops, oracle, tmp_path):
 REL_MFMA = 2e-3   # fp16 tiles into MFMA, fp32 accumulate
 
 
+@pytest.mark.parametrize("n_heads,n_kv,ctx,B", [(2, 2, 300, 37), (8, 2, 700, 64), (8, 1, 95, 13), (4, 4, 1029, 130)],
+                         ids=["mha", "gqa4_two_tiles_per_wave", "gqa8_short", "mha_deep_ragged"])
+def test_mfma_prefill_chunk_behind_long_cache(ops, oracle, n_heads, n_kv, ctx, B):
+    """A prefill chunk in the matrix-core mode behind a long synthetic cache: its attention runs over
+    many key tiles per wave, chunk sizes and positions that are not multiples of a tile, 1-8 query heads per
+    kv head.  Checked through what depends on it: the cache rows of the second layer and the next logits."""
+    from llama2_rs import _lib
+    dims = ck.Dims(dim=128 * n_heads, hidden_dim=512, n_layers=2, n_heads=n_heads, n_kv_heads=n_kv,
+                   vocab_size=300, seq_len=ctx + B + 8, group_size=128)
+    img = ck.synth_weights_image(dims, seed=9)
+    m = ops.Model(img, dims)
+    o = oracle.Model(img, dims)
+    m.set_prefill_mode(_lib.PREFILL_MFMA)
+    o.new_state()
+    m.fill_kv_synthetic(0, ctx, seed=4)
+    ko, vo = o.kv_cache()
+    for l in range(dims.n_layers):
+        k, v = m.read_kv(l, 0, ctx)
+        ko[l, :ctx] = k
+        vo[l, :ctx] = v
+    rng = np.random.default_rng(B)
+    toks = rng.integers(0, dims.vocab_size, size=B).astype(np.int32)
+    poss = np.arange(ctx, ctx + B, dtype=np.int32)
+    m.forward(toks, poss)
+    o.transformer(toks, poss)
+    k, v = m.read_kv(1, ctx, B)
+    # observed: 1-2e-3 on the rows (the fp16 rounding of the projections), 1-3e-5 on the logits
+    assert nrel(k, ko[1, ctx:ctx + B]) < 2.5 * REL_MFMA
+    assert nrel(v, vo[1, ctx:ctx + B]) < 2.5 * REL_MFMA
+    got = m.forward([7], [ctx + B])
+    want = o.transformer([7], [ctx + B])
+    assert nrel(got, want) < 0.25 * REL_MFMA
+    m.close()
+    o.close()
+
+
 @pytest.mark.parametrize("dims,B", [(TINY_GQA, 5), (MID, 33), (MID, 128)], ids=["gqa_g128_b5", "g32_b33", "g32_b128"])
 def test_mfma_prefill_operator_and_forward(ops, oracle, dims, B):
     """The dequant->fp16->MFMA form of QLinear::matvec<B> and of transformer<B> (B > 1)."""
