@@ -675,6 +675,8 @@ extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
     if (mode == L2_PREFILL_MFMA && m->d.group_size == 0)
         return l2_fail(L2_ERR_ARG, "the MFMA prefill path is the quantised model's");
     const int G = m->d.group_size;
+    if (mode == L2_PREFILL_MFMA && m->head_size != 128)
+        return l2_fail(L2_ERR_ARG, "the MFMA prefill path is built for heads of 128 (this model: %d)", m->head_size);
     if (mode == L2_PREFILL_MFMA && !(q4_gemm_supports(m->d.dim, m->d.dim, G) && q4_gemm_supports(m->d.hidden_dim, m->kv_dim, G) &&
                                      q4_gemm_supports(m->d.dim, m->d.hidden_dim, G)))
         return l2_fail(L2_ERR_ARG, "the MFMA prefill path needs dim and hidden_dim to be multiples of 128 (of 2 groups for "
@@ -1208,21 +1210,20 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
         t.inv[0] = m->q[L2_WQ][0].inv_index, t.inv[1] = m->q[L2_WK][0].inv_index, t.inv[2] = m->q[L2_WV][0].inv_index;
         t.out[0] = m->xq, t.out[1] = m->xk, t.out[2] = m->xv;
         L2_TRY(embed_launch(m->x, m->tok_emb, m->dtok, dim, B, t, m->amax, st));
+        // the first layer's inputs; every later layer gets them from the kernel that ends the layer before
+        L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
+        PrepList P{};
+        P.n_mats = 3;
+        P.out[0] = m->h16a, P.x[0] = m->xq, P.wn[0] = m->dwn + 0 * (size_t)dim;
+        P.out[1] = m->h16b, P.x[1] = m->xk, P.wn[1] = m->dwn + 1 * (size_t)dim;
+        P.out[2] = m->h16c, P.x[2] = m->xv, P.wn[2] = m->dwn + 2 * (size_t)dim;
+        L2_TRY(prep_f16_multi_launch(P, dim, B, st));
     }
     for (int l = 0; l < L; l++) {
         const DevQLinear &wq = m->q[L2_WQ][l], &wk = m->q[L2_WK][l], &wv = m->q[L2_WV][l],
                          &wo = m->q[L2_WO][l], &w1 = m->q[L2_W1][l], &w2 = m->q[L2_W2][l],
                          &w3 = m->q[L2_W3][l];
-        const float *wn = m->dwn + (size_t)l * 5 * dim;
-        L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
-        {
-            PrepList P{};
-            P.n_mats = 3;
-            P.out[0] = m->h16a, P.x[0] = m->xq, P.wn[0] = wn + 0 * (size_t)dim;
-            P.out[1] = m->h16b, P.x[1] = m->xk, P.wn[1] = wn + 1 * (size_t)dim;
-            P.out[2] = m->h16c, P.x[2] = m->xv, P.wn[2] = wn + 2 * (size_t)dim;
-            L2_TRY(prep_f16_multi_launch(P, dim, B, st));
-        }
+        RopeKvArgs R{};
         {
             Q4Launch Q = launch_of(wq, B, m->rms_eps);
             Q.m[0] = mat_of(wq, nullptr, nullptr, m->qv);
@@ -1230,32 +1231,27 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
             Q.m[2] = mat_of(wv, nullptr, nullptr, m->vv);
             Q.n_mats = 3;
             XhList X{{m->h16a, m->h16b, m->h16c}};
-            L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st));
+            // partial tiles; the kernel that adds them also applies the rms scale, RoPE and the cache write
+            L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st, &R.KS));
         }
         float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
         float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
-        L2_TRY(rope_kv_launch(m->qv, m->kv, m->vv, m->dpos, m->rope_cos, m->rope_sin, kc, vc, d.n_heads,
-                              d.n_kv_heads, m->head_size, B, st));
+        R.ws = m->gemm_ws, R.B = B, R.ss = m->ssb, R.pos = m->dpos, R.cos_t = m->rope_cos, R.sin_t = m->rope_sin;
+        R.q = m->qv, R.kcache = kc, R.vcache = vc, R.n_heads = d.n_heads, R.n_kv_heads = d.n_kv_heads;
+        L2_TRY(gemm_rope_kv_launch(R, st));
         L2_TRY(attention_launch(nullptr, m->h16a, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
                                 m->head_size, max_pos, B, st));
-        {
+        {   // wo: partial tiles, then residual + rms scale + the fp16 inputs of w1 and w3 in one kernel
             Q4Launch Q = launch_of(wo, B, 0.f);
             Q.m[0] = mat_of(wo, nullptr, nullptr, m->x);
-            Q.e.kind = Q4_EPI_RESIDUAL;
-            Q.e.res = m->x;
-            Q.e.n_scatter = 2;
-            Q.e.sc_idx[0] = w1.inv_index, Q.e.sc_out[0] = m->x1;
-            Q.e.sc_idx[1] = w3.inv_index, Q.e.sc_out[1] = m->x3;
             XhList X{{m->h16a, nullptr, nullptr}};
-            L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
-        }
-        L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
-        {
-            PrepList P{};
-            P.n_mats = 2;
-            P.out[0] = m->h16a, P.x[0] = m->x1, P.wn[0] = wn + 3 * (size_t)dim;
-            P.out[1] = m->h16b, P.x[1] = m->x3, P.wn[1] = wn + 4 * (size_t)dim;
-            L2_TRY(prep_f16_multi_launch(P, dim, B, st));
+            ResNormPrep R{};
+            L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st, &R.KS));
+            R.ws = m->gemm_ws, R.B = B, R.out = dim, R.res = m->x, R.x = m->x, R.ss = m->ssb, R.eps = m->rms_eps;
+            R.n = 2, R.wn = m->rms_ffn + (size_t)l * dim;
+            R.inv[0] = w1.inv_index, R.out_h[0] = m->h16a;
+            R.inv[1] = w3.inv_index, R.out_h[1] = m->h16b;
+            L2_TRY(gemm_residual_norm_prep_launch(R, st));
         }
         {
             Q4Launch Q = launch_of(w1, B, m->rms_eps);
@@ -1269,16 +1265,21 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
         {
             Q4Launch Q = launch_of(w2, B, 0.f);
             Q.m[0] = mat_of(w2, nullptr, nullptr, m->x);
-            Q.e.kind = Q4_EPI_RESIDUAL;
-            Q.e.res = m->x;
-            if (l + 1 < L) {
-                Q.e.n_scatter = 3;
-                Q.e.sc_idx[0] = m->q[L2_WQ][l + 1].inv_index, Q.e.sc_out[0] = m->xq;
-                Q.e.sc_idx[1] = m->q[L2_WK][l + 1].inv_index, Q.e.sc_out[1] = m->xk;
-                Q.e.sc_idx[2] = m->q[L2_WV][l + 1].inv_index, Q.e.sc_out[2] = m->xv;
-            }
             XhList X{{m->h16a, nullptr, nullptr}};
-            L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
+            if (l + 1 < L) { // the same kernel hands the next layer its q, k and v inputs
+                ResNormPrep R{};
+                L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st, &R.KS));
+                R.ws = m->gemm_ws, R.B = B, R.out = dim, R.res = m->x, R.x = m->x, R.ss = m->ssb, R.eps = m->rms_eps;
+                R.n = 3, R.wn = m->rms_att + (size_t)(l + 1) * dim;
+                R.inv[0] = m->q[L2_WQ][l + 1].inv_index, R.out_h[0] = m->h16a;
+                R.inv[1] = m->q[L2_WK][l + 1].inv_index, R.out_h[1] = m->h16b;
+                R.inv[2] = m->q[L2_WV][l + 1].inv_index, R.out_h[2] = m->h16c;
+                L2_TRY(gemm_residual_norm_prep_launch(R, st));
+            } else {
+                Q.e.kind = Q4_EPI_RESIDUAL;
+                Q.e.res = m->x;
+                L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
+            }
         }
     }
     return L2_OK;

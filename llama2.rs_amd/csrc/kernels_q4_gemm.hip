@@ -108,7 +108,7 @@ constexpr int kGemmXP = 2;
 
 template <int G, int NB, int KSTEP>
 __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
-                                                      float *__restrict__ ws, int KS) {
+                                                      float *__restrict__ ws, int KS, int partials) {
     Q4G_STAMP(0);
     constexpr int PW = kGemmPW, XP = kGemmXP;
     constexpr int W = KSTEP / 64;        // sub-steps of 64 k per K step
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             const int o = obase + oc;
             if (t >= B || o >= n_out) continue;
             const size_t row = (size_t)t * n_out;
-            if (KS > 1) { // partial tile of this K slice
+            if (KS > 1 || partials) { // partial tile of this K slice
                 *reinterpret_cast<float4 *>(ws + ws_base + ((size_t)ks * B + t) * n_out + o) = v;
                 continue;
             }
@@ -416,6 +416,113 @@ __global__ __launch_bounds__(256) void q4_gemm_reduce_kernel(const Q4Launch L, c
     }
 }
 
+// What follows a residual projection (wo, w2) of a chunk, in one kernel instead of three: add the KS partial
+// tiles in slice order and the residual (src/models.rs:263-264, 283-285), store the new residual stream,
+// take its rms scale (src/models.rs:55-60), and hand fp16 copies times the norm weight to up to three
+// consumers, each in its own act-order and in the pair-interleaved order the GEMM reads.
+// One block of 1024 threads per token, four outputs per thread and trip; every load of a trip (residual,
+// partial tiles, the consumers' indices, the norm weight) goes out before the first use.
+__global__ __launch_bounds__(1024) void gemm_residual_norm_prep_kernel(const ResNormPrep A) {
+    __shared__ float red[16];
+    extern __shared__ _Float16 perm_h[]; // [consumer][out]: the token's row in each consumer's order
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int n4 = A.out >> 2;
+    const size_t row = (size_t)t * A.out;
+    const size_t slice = (size_t)A.B * A.out;
+    float sq = 0.f;
+    for (int i4 = tid; i4 < n4; i4 += 1024) {
+        const float *p = A.ws + row + 4 * i4;
+        float4 v = *reinterpret_cast<const float4 *>(A.res + row + 4 * i4);
+        float4 part[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) part[ks] = *reinterpret_cast<const float4 *>(p + min(ks, A.KS - 1) * slice);
+        int4 idx[3];
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+            idx[c] = *reinterpret_cast<const int4 *>((c < A.n ? A.inv[c] : A.inv[0]) + 4 * i4);
+        const float4 g = *reinterpret_cast<const float4 *>(A.wn + 4 * i4); // one norm weight for all consumers
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++)
+            if (ks < A.KS) a.x += part[ks].x, a.y += part[ks].y, a.z += part[ks].z, a.w += part[ks].w;
+        v.x += a.x, v.y += a.y, v.z += a.z, v.w += a.w;
+        *reinterpret_cast<float4 *>(A.x + row + 4 * i4) = v;
+        sq = fmaf(v.x, v.x, sq), sq = fmaf(v.y, v.y, sq), sq = fmaf(v.z, v.z, sq), sq = fmaf(v.w, v.w, sq);
+        const _Float16 vals[4] = {(_Float16)(v.x * g.x), (_Float16)(v.y * g.y), (_Float16)(v.z * g.z), (_Float16)(v.w * g.w)};
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            if (c >= A.n) continue;
+            const int id[4] = {idx[c].x, idx[c].y, idx[c].z, idx[c].w};
+            // the permutation happens in LDS: the global stores below are whole 16-byte pieces
+#pragma unroll
+            for (int e = 0; e < 4; e++) perm_h[c * A.out + h16_slot(id[e])] = vals[e];
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+    if ((tid & 63) == 0) red[tid >> 6] = sq;
+    __syncthreads();
+    if (tid == 0) {
+        float s = 0.f;
+        for (int w = 0; w < 16; w++) s += red[w];
+        s /= (float)A.out;
+        s += A.eps;
+        A.ss[t] = 1.0f / sqrtf(s);
+    }
+    const int n8 = A.out >> 3;
+    for (int i = tid; i < A.n * n8; i += 1024) {
+        const int c = i / n8, j8 = i - c * n8;
+        reinterpret_cast<uint4 *>(reinterpret_cast<_Float16 *>(A.out_h[c]) + row)[j8] =
+            reinterpret_cast<const uint4 *>(perm_h + (size_t)c * A.out)[j8];
+    }
+}
+
+// What follows the q|k|v projection of a chunk, in one kernel instead of two: add the KS partial tiles of
+// the three matrices in slice order, apply the token's rms scale, rotate q and k (src/models.rs:100-129: the
+// second half of a head uses the first half's ROTATED value), write q back and k and v into the cache rows
+// of the tokens' positions (:236-249).  One block per token; thread -> (head, i < 64).
+__global__ __launch_bounds__(1024) void gemm_rope_kv_kernel(const RopeKvArgs A) {
+    constexpr int HS = 128, HALF = 64;
+    const int b = blockIdx.x;
+    const int dim = A.n_heads * HS, kv_dim = A.n_kv_heads * HS;
+    const int p = A.pos[b];
+    const float ss = A.ss[b];
+    const float *ct = A.cos_t + (size_t)p * HALF, *st = A.sin_t + (size_t)p * HALF;
+    const float *wq = A.ws + (size_t)b * dim;
+    const float *wk = A.ws + (size_t)A.KS * A.B * dim + (size_t)b * kv_dim;
+    const float *wv = wk + (size_t)A.KS * A.B * kv_dim;
+    const size_t sq = (size_t)A.B * dim, sk = (size_t)A.B * kv_dim;
+    float *kc = A.kcache + (size_t)p * kv_dim, *vc = A.vcache + (size_t)p * kv_dim;
+    for (int idx = threadIdx.x; idx < A.n_heads * HALF; idx += 1024) {
+        const int h = idx >> 6, i = idx & 63;
+        const float c = ct[i], s = st[i];
+        float qa = 0.f, qb = 0.f, ka = 0.f, kb = 0.f;
+        const bool has_k = h < A.n_kv_heads;
+        for (int ks = 0; ks < A.KS; ks++) {
+            qa += wq[ks * sq + h * HS + i];
+            qb += wq[ks * sq + h * HS + i + HALF];
+            if (has_k) {
+                ka += wk[ks * sk + h * HS + i];
+                kb += wk[ks * sk + h * HS + i + HALF];
+            }
+        }
+        qa *= ss, qb *= ss;
+        const float first = qa * c - qb * s;
+        A.q[(size_t)b * dim + h * HS + i] = first;
+        A.q[(size_t)b * dim + h * HS + i + HALF] = qb * c + first * s;
+        if (has_k) {
+            ka *= ss, kb *= ss;
+            const float kf = ka * c - kb * s;
+            kc[h * HS + i] = kf;
+            kc[h * HS + i + HALF] = kb * c + kf * s;
+        }
+    }
+    for (int i = threadIdx.x; i < kv_dim; i += 1024) {
+        float v = 0.f;
+        for (int ks = 0; ks < A.KS; ks++) v += wv[ks * sk + i];
+        vc[i] = v * ss;
+    }
+}
+
 // fp32 [B][n] (already in the consumer's g_index order) -> fp16 [B][n], times the
 // norm weight if given, with the (0,4,1,5,2,6,3,7) interleave inside every 8.
 __global__ void prep_f16_kernel(const PrepList P, int n) {
@@ -464,23 +571,45 @@ __global__ __launch_bounds__(256) void rms_scale_kernel(float *ss, const float *
 }
 
 // silu gate (src/models.rs:92-98) for a chunk: out[b][scatter[i]] = silu(a[b][i]) * c[b][i]
-__global__ void silu_scatter_kernel(float *out, _Float16 *out_h, const float *a, const float *c,
-                                    const int32_t *scatter, int n) {
+__global__ void silu_scatter_kernel(float *out, const float *a, const float *c, const int32_t *scatter, int n) {
     const int b = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float s = a[(size_t)b * n + i];
     s = s * (1.0f / (1.0f + expf(-s)));
     s = s * c[(size_t)b * n + i];
-    const int j = scatter ? scatter[i] : i;
-    if (out_h)
-        out_h[(size_t)b * n + h16_slot(j)] = (_Float16)s;
-    else
-        out[(size_t)b * n + j] = s;
+    out[(size_t)b * n + (scatter ? scatter[i] : i)] = s;
+}
+
+// The same gate handing fp16 to the next GEMM: one block per token permutes the token's row in LDS (the
+// consumer's act-order, pair-interleaved), so that the global stores are whole 16-byte pieces.
+__global__ __launch_bounds__(1024) void silu_scatter_f16_kernel(_Float16 *__restrict__ out_h, const float *__restrict__ a,
+                                                                const float *__restrict__ c,
+                                                                const int32_t *__restrict__ scatter, int n) {
+    extern __shared__ _Float16 perm_row[]; // [n]
+    const size_t row = (size_t)blockIdx.x * n;
+    const int tid = threadIdx.x;
+    for (int i4 = tid; i4 < (n >> 2); i4 += 1024) {
+        const float4 x = *reinterpret_cast<const float4 *>(a + row + 4 * i4);
+        const float4 y = *reinterpret_cast<const float4 *>(c + row + 4 * i4);
+        const int4 id = *reinterpret_cast<const int4 *>(scatter + 4 * i4);
+        const float xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
+        const int ids[4] = {id.x, id.y, id.z, id.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float s = xs[e];
+            s = s * (1.0f / (1.0f + expf(-s)));
+            perm_row[h16_slot(ids[e])] = (_Float16)(s * ys[e]);
+        }
+    }
+    __syncthreads();
+    for (int j8 = tid; j8 < (n >> 3); j8 += 1024)
+        reinterpret_cast<uint4 *>(out_h + row)[j8] = reinterpret_cast<const uint4 *>(perm_row)[j8];
 }
 
 template <int G>
-int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st) {
+int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st,
+                  int *ks_out) {
     int total = 0;
     long rows = 0;
     for (int i = 0; i < L.n_mats; i++) {
@@ -508,11 +637,15 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     // the activation buffers, or the four output staging tiles of the epilogue (32 x 36 floats per wave)
     const size_t lds = std::max((size_t)2 * TN * (KSTEP + kXPad) * sizeof(_Float16), (size_t)4 * 32 * 36 * sizeof(float));
     switch (NB) {
-        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS); break;
-        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS); break;
+        case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS, ks_out != nullptr); break;
+        case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS, ks_out != nullptr); break;
         default: return l2_fail(L2_ERR_ARG, "q4 gemm: token tile");
     }
     L2_HIP(hipGetLastError());
+    if (ks_out) { // the caller's own kernel adds the partial tiles
+        *ks_out = KS;
+        return L2_OK;
+    }
     if (KS > 1) {
         hipLaunchKernelGGL(q4_gemm_reduce_kernel, dim3((unsigned)((rows + 1023) / 1024), B), dim3(256), 0, st, L, ss, ws, KS);
         L2_HIP(hipGetLastError());
@@ -523,7 +656,7 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
 } // namespace
 
 int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, float *ws, size_t ws_floats,
-                   hipStream_t st) {
+                   hipStream_t st, int *ks_out) {
     if (L.n_mats < 1 || L.n_mats > 3) return l2_fail(L2_ERR_ARG, "q4 gemm: n_mats=%d", L.n_mats);
     if (L.in % 128 != 0 || L.in % L.group_size != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: in=%d must be a multiple of 128", L.in);
     if (L.group_size >= 64 && (L.in / L.group_size) % 2 != 0)
@@ -532,9 +665,9 @@ int q4_gemm_launch(Q4Launch &L, const XhList &xh_list_dev, const float *ss, floa
         if (L.m[i].out % 32 != 0) return l2_fail(L2_ERR_ARG, "q4 gemm: out=%d must be a multiple of 32", L.m[i].out);
     if (L.pair) return l2_fail(L2_ERR_ARG, "q4 gemm: pair launches are not supported");
     switch (L.group_size) {
-        case 32: return launch_gemm_g<32>(L, xh_list_dev, ss, ws, ws_floats, st);
-        case 64: return launch_gemm_g<64>(L, xh_list_dev, ss, ws, ws_floats, st);
-        case 128: return launch_gemm_g<128>(L, xh_list_dev, ss, ws, ws_floats, st);
+        case 32: return launch_gemm_g<32>(L, xh_list_dev, ss, ws, ws_floats, st, ks_out);
+        case 64: return launch_gemm_g<64>(L, xh_list_dev, ss, ws, ws_floats, st, ks_out);
+        case 128: return launch_gemm_g<128>(L, xh_list_dev, ss, ws, ws_floats, st, ks_out);
     }
     return l2_fail(L2_ERR_ARG, "q4 gemm: group size %d", L.group_size);
 }
@@ -566,8 +699,44 @@ int rms_scale_launch(float *ss, const float *x, float eps, int dim, int B, hipSt
 
 int silu_scatter_launch(float *out, void *out_f16, const float *a, const float *c, const int32_t *scatter, int n,
                         int B, hipStream_t st) {
-    hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, (_Float16 *)out_f16, a, c,
-                       scatter, n);
+    if (out_f16) {
+        if (!scatter || n % 8 || (size_t)n * 2 > 60 * 1024)
+            return l2_fail(L2_ERR_ARG, "silu gate (fp16): n=%d needs a permutation and at most 60 KB of LDS", n);
+        static size_t raised = 48 * 1024;
+        if ((size_t)n * 2 > raised) {
+            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(silu_scatter_f16_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, n * 2));
+            raised = (size_t)n * 2;
+        }
+        hipLaunchKernelGGL(silu_scatter_f16_kernel, dim3(B), dim3(1024), (size_t)n * 2, st, (_Float16 *)out_f16, a, c, scatter, n);
+    } else {
+        hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, a, c, scatter, n);
+    }
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int gemm_residual_norm_prep_launch(const ResNormPrep &A, hipStream_t st) {
+    if (A.KS < 1 || A.KS > 8 || A.out % 4 || A.n < 0 || A.n > 3)
+        return l2_fail(L2_ERR_ARG, "residual epilogue: %d slices, %d outputs, %d consumers", A.KS, A.out, A.n);
+    if (A.n == 0) return l2_fail(L2_ERR_ARG, "residual epilogue: no consumer");
+    const size_t lds = (size_t)A.n * A.out * sizeof(_Float16);
+    if (A.out % 8 || lds > 60 * 1024) return l2_fail(L2_ERR_ARG, "residual epilogue: %d outputs x %d consumers", A.out, A.n);
+    static size_t raised = 48 * 1024;
+    if (lds > raised) {
+        L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_residual_norm_prep_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = lds;
+    }
+    hipLaunchKernelGGL(gemm_residual_norm_prep_kernel, dim3(A.B), dim3(1024), lds, st, A);
+    L2_HIP(hipGetLastError());
+    return L2_OK;
+}
+
+int gemm_rope_kv_launch(const RopeKvArgs &A, hipStream_t st) {
+    if (A.KS < 1 || A.KS > 8 || A.B < 1 || A.n_heads < A.n_kv_heads)
+        return l2_fail(L2_ERR_ARG, "q|k|v epilogue: %d slices, %d tokens", A.KS, A.B);
+    hipLaunchKernelGGL(gemm_rope_kv_kernel, dim3(A.B), dim3(1024), 0, st, A);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }

@@ -121,7 +121,36 @@ struct XhList {
 // Y = X W^T for a chunk of L.batch tokens; ss (per token, may be null) scales the rows of Y.
 // Epilogues as in the matvec (no pair launches).  ws: workspace of ws_floats floats for split-K partial
 // tiles (the launcher uses as many K slices as fit).
-int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st);
+// ks_out given: the kernel leaves its K slices as partial tiles [KS][B][out] in ws (also when KS is 1), no
+// reduction is launched, and *ks_out says how many there are.
+int q4_gemm_launch(Q4Launch &L, const XhList &xh, const float *ss, float *ws, size_t ws_floats, hipStream_t st,
+                   int *ks_out = nullptr);
+
+struct ResNormPrep {
+    const float *ws;   // partial tiles [KS][B][out] of one matrix
+    int KS, B, out;
+    const float *res;  // [B][out] residual stream in
+    float *x;          // [B][out] residual stream out (may be res)
+    float *ss;         // [B] rms scale of the new residual stream
+    float eps;
+    int n;             // consumers (1..3)
+    const int32_t *inv[3]; // inverse act-order permutation of each consumer
+    const float *wn;       // [out] norm weight of the consumers' rmsnorm, in the order of the residual stream
+    void *out_h[3];        // [B][out] fp16, pair-interleaved, in each consumer's order
+};
+int gemm_residual_norm_prep_launch(const ResNormPrep &A, hipStream_t st);
+
+struct RopeKvArgs {
+    const float *ws;   // partial tiles of q, k, v laid end to end: [KS][B][dim], [KS][B][kv_dim], [KS][B][kv_dim]
+    int KS, B;
+    const float *ss;   // [B] rms scale of the layer's input
+    const int32_t *pos;
+    const float *cos_t, *sin_t;
+    float *q;          // [B][dim] out
+    float *kcache, *vcache; // the layer's cache: rows [pos][kv_dim]
+    int n_heads, n_kv_heads; // head size 128
+};
+int gemm_rope_kv_launch(const RopeKvArgs &A, hipStream_t st);
 bool q4_gemm_supports(int in, int out, int group_size);
 // out_f16[b][j'] = fp16(x[b][j] * (wn ? wn[j] : 1)), j' = j with the order (0,4,1,5,2,6,3,7) inside every 8.
 int prep_f16_launch(void *out_f16, const float *x, const float *wn, int n, int B, hipStream_t st);
