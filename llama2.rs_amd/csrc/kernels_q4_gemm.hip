@@ -118,6 +118,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     constexpr bool SA = G >= 64; // scale after the group's partial sum
     extern __shared__ _Float16 xs[]; // [2][TN][kXRow]
     __shared__ float gsc[2][kGemmPW][128]; // fp32 scales of the block's 128 rows, PW groups at a time
+    __shared__ int32_t zsc[2][kGemmPW][16]; // their packed zero points: one word per 8 rows and group
     const int in = L.in;
     const int n_k = in / KSTEP; // K iterations
 
@@ -175,11 +176,12 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
 #pragma unroll
         for (int sw = 0; sw < W; sw++)
             d.w[sw] = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc * (2 * W) + 2 * sw + h) << 4);
-        d.z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
-        if constexpr (SA)
-            d.s = 0.f;
-        else
+        if constexpr (SA) {
+            d.z = 0, d.s = 0.f; // scale-after form: zero points and scales travel by the block, PW groups at a time
+        } else {
+            d.z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
             d.s = ld_at<float>(sc_base, (uint32_t)(orow * groups + g) << 2);
+        }
     };
     // Scale-after form: one 8-byte load per thread and PW K steps (a K step is a group there) instead of
     // one scattered 4-byte load per thread and step.  Block j of PW groups starts at group kit0 + PW * j;
@@ -193,6 +195,14 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
         gsc[j & 1][2 * ghalf][tid & 127] = v.x;
         gsc[j & 1][2 * ghalf + 1][tid & 127] = v.y;
     };
+    // zero points of the same PW groups: 16 row groups x PW words per block; every wave fetches the same 64
+    // words (no load under a branch), lane -> (row group lane / 4, group lane % 4)
+    const int zrg = min(rb * 16 + (lane >> 2), (n_out - 1) >> 3);
+    auto fetch_zs = [&](int j) {
+        const int ge = min(kit0 + PW * j + (lane & 3), groups - 1);
+        return ld_at<int32_t>(qz_base, (uint32_t)(zrg * groups + ge) << 2);
+    };
+    auto store_zs = [&](int j, const int32_t v) { zsc[j & 1][lane & 3][lane >> 2] = v; };
     // staging map: thread -> (token, 16-byte segment) x (TN*8/256) pieces
     constexpr int SEGS = KSTEP / 8; // 16-byte segments per token and K step
     constexpr int PIECES = TN * SEGS / 256;
@@ -223,25 +233,27 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     XStage xr[XP];
     WStage wr[PW];
     float2 gs2 = make_float2(0.f, 0.f);
-    if constexpr (SA) gs2 = fetch_gs(0);
+    int32_t zs2 = 0;
+    if constexpr (SA) gs2 = fetch_gs(0), zs2 = fetch_zs(0);
 #pragma unroll
     for (int j = 0; j < XP; j++) fetch_x(kit0 + j, xr[j]);
 #pragma unroll
     for (int j = 0; j < PW; j++) fetch_w(kit0 + j, wr[j]);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the loop's waits then reflect its own order only
     store_x(0, xr[0]);
-    if constexpr (SA) store_gs(0, gs2);
+    if constexpr (SA) store_gs(0, gs2), store_zs(0, zs2);
     __syncthreads();
     Q4G_STAMP(1);
 
-    for (int base = 0; base < n_it; base += PW) {
-#pragma unroll
-        for (int u = 0; u < PW; u++) {
-            if (base + u >= n_it) break; // uniform
-            const int kit = kit0 + base + u;
-            const int buf = (base + u) & 1; // PW is even: the parity of u
+    // One K step; u = step % PW indexes the register rings (a compile-time constant where it is called).
+    auto k_step = [&](const int stepi, const int u) __attribute__((always_inline)) {
+        {
+            const int base = stepi - u;
+            const int kit = kit0 + stepi;
+            const int buf = u & 1; // PW is even: the parity of the step
             // this step's weights -> registers of their own, then refill the slot
-            const int zn = (wr[u].z >> (4 * (orow & 7))) & 15;
+            const int zword = SA ? zsc[(stepi / PW) & 1][u][(wave * 32 + r) >> 3] : wr[u].z;
+            const int zn = (zword >> (4 * (orow & 7))) & 15;
             DequantConsts dc;
             dc.mask_lo = 0x000F000Fu, dc.mask_hi = 0x00F000F0u, dc.magic = 0x64006400u;
             const _Float16 off = (_Float16)(-(1024.0f + (float)(zn + 1)));
@@ -257,11 +269,18 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                 wd[sw][0] = wr[u].w[sw].x, wd[sw][1] = wr[u].w[sw].y, wd[sw][2] = wr[u].w[sw].z, wd[sw][3] = wr[u].w[sw].w;
                 asm volatile("" : "+v"(wd[sw][0]), "+v"(wd[sw][1]), "+v"(wd[sw][2]), "+v"(wd[sw][3])::"memory");
             }
+            // The ring slot stays in its own registers up to here (the copies above live elsewhere), so the
+            // refill can land in them: otherwise the copy takes the slot's registers over, the refill goes to
+            // fresh ones and is copied back at the loop's end, behind a wait for the load just issued.
+#pragma unroll
+            for (int sw = 0; sw < W; sw++)
+                asm volatile("" : "+v"(wr[u].w[sw].x), "+v"(wr[u].w[sw].y), "+v"(wr[u].w[sw].z), "+v"(wr[u].w[sw].w));
+            if constexpr (!SA) asm volatile("" : "+v"(wr[u].z));
             __builtin_amdgcn_sched_barrier(0);
             fetch_w(kit + PW, wr[u]);
             fetch_x(kit + XP, xr[u % XP]);
             if constexpr (SA)
-                if (u == 0) gs2 = fetch_gs(base / PW + 1); // the next PW groups' scales
+                if (u == 0) gs2 = fetch_gs(base / PW + 1), zs2 = fetch_zs(base / PW + 1); // the next PW groups' scales and zeros
             __builtin_amdgcn_sched_barrier(0);
             const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
             // W * 4 steps of 16 k.  The operands of step i + 1 (two LDS reads per token tile, the
@@ -305,13 +324,24 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                             accg[nb][4 * q + e] = 0.f;
                         }
                 }
-                if (u == PW - 1) store_gs(base / PW + 1, gs2); // fetched at the first step of this round
+                if (u == PW - 1) store_gs(base / PW + 1, gs2), store_zs(base / PW + 1, zs2); // fetched at the round's first step
             }
             // the next step's activation tile was fetched XP - 1 steps ago
             store_x(buf ^ 1, xr[(u + 1) % XP]);
             __syncthreads();
         }
+    };
+    // Whole rounds of PW steps in the loop, the remaining steps straight-line after it: an exit from the
+    // middle of the unrolled body makes the compiler copy ring registers at the loop's end, and every copy
+    // waits for its load, which drains the prefetch once per round.
+    const int n_full = n_it / PW, n_rem = n_it - n_full * PW;
+    for (int bi = 0; bi < n_full; bi++) {
+#pragma unroll
+        for (int u = 0; u < PW; u++) k_step(bi * PW + u, u);
     }
+#pragma unroll
+    for (int u = 0; u < PW - 1; u++)
+        if (u < n_rem) k_step(n_full * PW + u, u);
 
     Q4G_STAMP(2);
     // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4.
