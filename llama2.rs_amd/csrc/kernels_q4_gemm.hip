@@ -277,11 +277,28 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                 asm volatile("" : "+v"(wr[u].w[sw].x), "+v"(wr[u].w[sw].y), "+v"(wr[u].w[sw].z), "+v"(wr[u].w[sw].w));
             if constexpr (!SA) asm volatile("" : "+v"(wr[u].z));
             __builtin_amdgcn_sched_barrier(0);
-            fetch_w(kit + PW, wr[u]);
-            fetch_x(kit + XP, xr[u % XP]);
-            if constexpr (SA)
-                if (u == 0) gs2 = fetch_gs(base / PW + 1), zs2 = fetch_zs(base / PW + 1); // the next PW groups' scales and zeros
-            __builtin_amdgcn_sched_barrier(0);
+            // The refills of this step (ring slot u of the weights, slot u % XP of the activations, once per
+            // round the next PW groups' scales and zero points) are issued one at a time between the MFMA
+            // steps below: a global load takes the wave hundreds of cycles to issue when the address unit is
+            // busy, and issued in one burst here those cycles stood in front of the first MFMA.
+            const int kc_w = min(kit + PW, kit1 - 1);
+            const uint32_t kb_x = (uint32_t)min(kit + XP, kit1 - 1) * (uint32_t)(KSTEP * 2);
+            constexpr int NL = W + 1 + PIECES + 1;
+            auto refill = [&](const int i) __attribute__((always_inline)) {
+                if (i < W) {
+                    wr[u].w[i] = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc_w * (2 * W) + 2 * i + h) << 4);
+                } else if (i == W) {
+                    if constexpr (!SA) {
+                        const int g = (kc_w * KSTEP + 32 * h) / G;
+                        wr[u].z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
+                        wr[u].s = ld_at<float>(sc_base, (uint32_t)(orow * groups + g) << 2);
+                    }
+                } else if (i < W + 1 + PIECES) {
+                    xr[u % XP].v[i - W - 1] = ld_at<uint4>(xh, xoff[i - W - 1] + kb_x);
+                } else if (SA && u == 0) {
+                    gs2 = fetch_gs(base / PW + 1), zs2 = fetch_zs(base / PW + 1);
+                }
+            };
             const _Float16 *xb = xs + (size_t)buf * TN * kXRow;
             // W * 4 steps of 16 k.  The operands of step i + 1 (two LDS reads per token tile, the
             // dequantised weights) are produced while the MFMAs of step i run: without this the
@@ -299,6 +316,8 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             produce(0, 0);
 #pragma unroll
             for (int step = 0; step < NSTEP; step++) {
+#pragma unroll
+                for (int i = step * NL / NSTEP; i < (step + 1) * NL / NSTEP; i++) refill(i);
                 if (step + 1 < NSTEP) produce(step + 1, (step + 1) & 1);
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
