@@ -482,8 +482,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(float *__restrict__ o
 // Wave w takes the key tiles w, w+8, ... of 32 cache rows each and keeps a running (m, l, O) of its own;
 // the block merges the eight at the end.  Per tile, with lane = (n = lane%32, h = lane/32):
 //   S^T = K Q^T      A: lane (key n, h) holds K[key][64h + s], B: lane (column n, h) holds Q[n][64h + s]
-//                    (the contraction index of MFMA step s and half h is d = 64h + s: each lane reads
-//                    256 contiguous bytes of its key row), 64 steps.
+//                    (the contraction index of MFMA step s and half h is d = 64h + s), 64 steps.  K reaches
+//                    that layout through the wave's LDS tile: loaded lane-per-row-half, a load instruction
+//                    touches 64 cache lines and the address unit becomes the bottleneck.
 //   C layout         lane (column n, h), register r -> key (r/4)*8 + 4h + r%4: a lane holds 16 scores of
 //                    ITS column, so the running maximum and sum are per-lane work plus one exchange
 //                    between the two halves.
@@ -513,14 +514,16 @@ __global__ __launch_bounds__(512) void attn_prefill_mfma_kernel(_Float16 *__rest
     const uint32_t row_bytes = (uint32_t)kv_dim * 4u;
     const int last_row = max_pos; // the last cache row written: loads clamp to it and wait for nothing
 
-    // K: this lane's half of its key row; V: the tile row by row, 16 bytes per lane and load.  Rows past
+    // K and V: the tile row by row, 16 bytes per lane and load (whole cache lines per instruction).  Rows past
     // the end re-read the last row (masked below), so the loads are unconditional.
     float4 kr[16], vr[16];
-    auto fetch_k = [&](int kt) {
-        const int tk = min(kt * TK + n, last_row);
-        const uint32_t off = __umul24(tk, row_bytes) + (uint32_t)(kvh * HS + 64 * h) * 4u;
+    auto fetch_k = [&](int kt) { // row by row like V: 32 lanes read one row's 512 bytes
 #pragma unroll
-        for (int i = 0; i < 16; i++) kr[i] = ld_at<float4>(kc, off + 16 * i);
+        for (int i = 0; i < 16; i++) {
+            const int f = i * 64 + lane;
+            const int tk = min(kt * TK + (f >> 5), last_row);
+            kr[i] = ld_at<float4>(kc, __umul24(tk, row_bytes) + (uint32_t)(kvh * HS + 4 * (f & 31)) * 4u);
+        }
     };
     auto fetch_v = [&](int kt) {
 #pragma unroll
@@ -572,23 +575,34 @@ __global__ __launch_bounds__(512) void attn_prefill_mfma_kernel(_Float16 *__rest
 #pragma unroll
         for (int r = 0; r < 16; r++) sacc[r] = 0.f;
         // the Q operands of steps 4i+4..4i+7 are read from LDS while the MFMAs of steps 4i..4i+3 run
-        float qv[2][4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) qv[0][e] = qst[(64 * h + e) * kQRow + n];
+        // K: the tile as loaded (row-wise, whole cache lines per load) -> the wave's LDS tile -> the A-operand
+        // layout (lane (key n, h) holds d = 64h .. 64h + 63); the next tile's keys go out meanwhile
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const float kk[4] = {kr[i].x, kr[i].y, kr[i].z, kr[i].w};
+            const int f = i * 64 + lane;
+            *reinterpret_cast<float4 *>(&vs[(f >> 5) * kVRow + 4 * (f & 31)]) = kr[i];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_k(kt + NWV);
+        __builtin_amdgcn_sched_barrier(0);
+        float qv[2][4];
+        float4 ka[2];
+#pragma unroll
+        for (int e = 0; e < 4; e++) qv[0][e] = qst[(64 * h + e) * kQRow + n];
+        ka[0] = *reinterpret_cast<const float4 *>(&vs[n * kVRow + 64 * h]);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float kk[4] = {ka[i & 1].x, ka[i & 1].y, ka[i & 1].z, ka[i & 1].w};
             if (i + 1 < 16) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) qv[(i + 1) & 1][e] = qst[(64 * h + 4 * (i + 1) + e) * kQRow + n];
+                ka[(i + 1) & 1] = *reinterpret_cast<const float4 *>(&vs[n * kVRow + 64 * h + 4 * (i + 1)]);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int e = 0; e < 4; e++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[e], qv[i & 1][e], sacc, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        fetch_k(kt + NWV); // the next tile's keys travel while this tile's softmax and P V run
-        __builtin_amdgcn_sched_barrier(0);
         // the V tile into the wave's own LDS region (the wave's LDS accesses execute in order)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
