@@ -149,8 +149,8 @@ struct RowData {
 
 // MODE 0: fp32 inner loop, x staged through LDS (rmsnorm prologue, several matrices, row pairs).
 // MODE 1: integer-dot inner loop, x staged and quantised in LDS.
-// MODE 2: fp32 inner loop, one matrix without rmsnorm: every lane loads its own 32 values of x
-//         straight into registers; no LDS staging, no barrier before the first row.
+// MODE 2: fp32 inner loop, one matrix without rmsnorm: every wave loads its own slice of x (coalesced)
+//         and turns it into the per-lane chunks through LDS of its own; no barrier before the first row.
 template <int G, int NWK, int S, bool PAIR, int MODE, int P>
 __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L) {
     constexpr bool IDOT = MODE == 1, DIRECT = MODE == 2;
@@ -224,9 +224,12 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     StageRegs xr[DIRECT ? 1 : NM];
     float4 xd[DIRECT ? 8 : 1];
     if constexpr (DIRECT) {
-        const float4 *xp = reinterpret_cast<const float4 *>(L.m[mi].x + (size_t)b * in) + cc * 8;
+        // this wave's 64 chunks of x, 1 KB per load instruction (whole cache lines); past the end the last
+        // 16 bytes are re-read and zeroed below
+        const float4 *xp = reinterpret_cast<const float4 *>(L.m[mi].x + (size_t)b * in);
+        const int n4 = in >> 2;
 #pragma unroll
-        for (int i = 0; i < 8; i++) xd[i] = xp[i];
+        for (int i = 0; i < 8; i++) xd[i] = xp[min(kslice * 512 + i * 64 + lane, n4 - 1)];
     } else {
 #pragma unroll
         for (int q = 0; q < NM; q++)
@@ -248,10 +251,20 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     float ss = 1.0f;
     const bool norm = !DIRECT && L.m[mi].wn != nullptr;
     if constexpr (DIRECT) {
+        // Turned through a region of LDS of the wave's own, from "lane l holds floats 4l..4l+3 of every 256"
+        // to "lane l holds its chunk's 32": no block barrier (a wave's LDS accesses execute in order).
+        float *xw = lds + wave * (64 * kChunkPad);
+        const int n4 = in >> 2;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int j4 = i * 64 + lane; // float4 index within the wave's slice
+            const float4 v = kslice * 512 + j4 < n4 ? xd[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4 *>(&xw[(j4 >> 3) * kChunkPad + (j4 & 7) * 4]) = v;
+        }
         float t = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const float4 v = has_chunk ? xd[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 v = *reinterpret_cast<const float4 *>(&xw[lane * kChunkPad + 4 * i]);
             x[0][4 * i + 0] = v.x;
             x[0][4 * i + 1] = v.y;
             x[0][4 * i + 2] = v.z;
@@ -524,7 +537,8 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     constexpr int NW = NWK * S;
     constexpr int TR = P * S;
     const int C = L.in / 32;
-    const size_t lds = MODE == 2 ? 0 : (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
+    const size_t lds = MODE == 2 ? (size_t)NW * 64 * kChunkPad * sizeof(float)
+                                 : (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
     if (lds + 8 * 1024 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
     int total = 0;
     const int rpb = plan_rows(L, NW, TR, lds, PAIR, &total);
@@ -553,8 +567,14 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
 template <int G, int MODE>
 int launch_sg(Q4Launch &L, hipStream_t stream) {
     const int nwk = (L.in / 32 + 63) / 64;
-    if constexpr (MODE == 2) {
-        if (!L.pair && nwk >= 9 && nwk <= 14) return launch_s<G, 14, 1, false, MODE>(L, stream);
+    if constexpr (MODE == 2) { // only the shapes q4_stream_launch sends here
+        if (!L.pair) switch (nwk) {
+            case 3:
+                if (plan_cost(L, 3, 5, 4, false) < plan_cost(L, 3, 4, 4, false)) return launch_s<G, 3, 5, false, MODE>(L, stream);
+                return launch_s<G, 3, 4, false, MODE>(L, stream);
+            case 7: return launch_s<G, 7, 2, false, MODE, 5>(L, stream);
+            case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, MODE>(L, stream);
+        }
     } else if (!L.pair) {
         switch (nwk) {
             case 1: return launch_s<G, 1, 4, false, MODE>(L, stream);
@@ -587,10 +607,14 @@ int q4_stream_launch(Q4Launch &L, hipStream_t stream) {
         const char *v = getenv("L2_Q4_IMPL");
         return !(v && !strcmp(v, "idot"));
     }();
-    // One matrix, no rmsnorm in front, and an input so long that its staging (over 64 KB of LDS per block)
-    // costs more than lanes fetching their own 128 bytes: x goes straight to registers.  For shorter inputs
-    // the strided 16-byte loads of that form were measured slower than the LDS staging (4096: 7.5 vs 5.9 us).
-    const bool direct = fp32_form && !L.pair && L.n_mats == 1 && L.m[0].wn == nullptr && L.in > 16384;
+    // One matrix and no rmsnorm in front: x can reach the registers through LDS of each wave's own instead
+    // of a block-wide staging with a barrier.  Measured per input width (cadence of the launch, block-wide
+    // against per-wave): 28672: 30.3 -> 28.6 us; 13824: 14.2 -> 13.2; 5120: 9.0 -> 7.7; but 11008: 9.0 -> 9.5,
+    // 8192: 11.6 -> 12.3, 4096 equal within the model.  The per-wave form is taken where it won: 3 and 7 waves
+    // per row, and inputs too long to stage block-wide beside a second block.
+    const int nwk = (L.in / 32 + 63) / 64;
+    const bool direct = fp32_form && !L.pair && L.n_mats == 1 && L.m[0].wn == nullptr &&
+                        (L.in > 16384 || nwk == 3 || nwk == 7);
     if (direct) {
         switch (L.group_size) {
             case 32: return launch_sg<32, 2>(L, stream);
