@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 # (each scaled by the reading of the plain copy kernel of known size in the same run):
 # the summaries are profiles/q4_matvec_<model>_decode_hbm_counters.txt.
 MEASURED_Q4_TRAFFIC_PER_LAYER = {
-    "7B": 49216073 + 2 * 18698448 + 24780114 + 235599 + 2 * 125403 + 265889,
+    "7B": 49226169 + 2 * 18683076 + 24774068 + 234963 + 2 * 125403 + 265887,
 }
 
 
