@@ -46,6 +46,7 @@ def test_kat_constant_cases(ops):
     (5120, 5120, 128, 1), (13824, 5120, 128, 2),
     (8192, 1024, 64, 1), (8192, 8192, 64, 1), (28672, 8192, 64, 1),
     (256, 64, 32, 3), (512, 40, 64, 1), (1024, 264, 128, 5),
+    (4160, 72, 32, 2), (12320, 40, 32, 1),   # rows of 3 and 7 waves with a ragged last wave
 ])
 def test_qmatvec_vs_oracle(ops, oracle, n_in, n_out, G, B):
     rng = np.random.default_rng(0)
