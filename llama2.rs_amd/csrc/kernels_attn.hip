@@ -63,7 +63,7 @@ template <int QG, int NWV>
 __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode A) {
     constexpr int NT = NWV * 64, TSTEP = NWV * 4;
     constexpr int HS = 128, HALF = 64;
-    constexpr int PD = QG >= 8 ? 2 : 4; // steps in flight (8 was measured slower at short contexts: coarser tiles)
+    constexpr int PD = QG >= 8 ? 2 : 4; // steps in flight and per pass through the phases (4 at 8 heads: over 256 registers, one block per CU, slower)
     __shared__ float qs[QG * HS];
     __shared__ float kvnew[2][HS];
     __shared__ float comb[NWV][QG][HS + 2];
@@ -185,25 +185,35 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
             for (int u = 0; u < PD; u++) fetch(tile * PD + u, pipe[u]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        // The tile's PD steps go through the phases together — all scores, one update of the running maxima,
+        // all weights and weighted sums — so that the dependent chains of one step (dot product, four
+        // cross-lane adds, exponential) interleave with those of the others: a block is often alone on its
+        // CU, one wave per SIMD, and nothing else fills the gaps between dependent instructions.
+        float v[PD][8];
+        float sc[PD][QG];
+        bool valid[PD];
+        float mt[QG];
+#pragma unroll
+        for (int j = 0; j < QG; j++) mt[j] = kNoScore;
 #pragma unroll
         for (int u = 0; u < PD; u++) {
             const int t = t0 + (tile * PD + u) * TSTEP + tl;
-            const bool valid = t < t1;
+            valid[u] = t < t1;
             const Step &d = pipe[u];
             float k[8] = {d.k0.x, d.k0.y, d.k0.z, d.k0.w, d.k1.x, d.k1.y, d.k1.z, d.k1.w};
-            float v[8] = {d.v0.x, d.v0.y, d.v0.z, d.v0.w, d.v1.x, d.v1.y, d.v1.z, d.v1.w};
+            const float vv[8] = {d.v0.x, d.v0.y, d.v0.z, d.v0.w, d.v1.x, d.v1.y, d.v1.z, d.v1.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[u][e] = vv[e];
             if (__any(t == pos)) { // once per block: the row of the new position comes from LDS, not from the cache
                 const bool is_new = t == pos;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     k[e] = is_new ? kvnew[0][ds * 8 + e] : k[e];
-                    v[e] = is_new ? kvnew[1][ds * 8 + e] : v[e];
+                    v[u][e] = is_new ? kvnew[1][ds * 8 + e] : v[u][e];
                 }
             }
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = valid ? v[e] : 0.f; // a row past the end may hold anything, NaN included
-            float sc[QG];
-            bool grow = false;
+            for (int e = 0; e < 8; e++) v[u][e] = valid[u] ? v[u][e] : 0.f; // a row past the end may hold anything, NaN included
 #pragma unroll
             for (int j = 0; j < QG; j++) {
                 float s = 0.f;
@@ -221,27 +231,33 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
                 s += dpp_xchg<0x4E>(s);
                 s += dpp_xchg<0x141>(s);
                 s += dpp_xchg<0x140>(s);
-                s = valid ? s * scale : kNoScore;
-                sc[j] = s;
-                grow |= s > m[j];
+                s = valid[u] ? s * scale : kNoScore;
+                sc[u][j] = s;
+                mt[j] = fmaxf(mt[j], s);
             }
-            if (__any(grow)) { // some row's maximum moves: rescale what was summed so far
+        }
+        bool grow = false;
 #pragma unroll
-                for (int j = 0; j < QG; j++) {
-                    const float m_new = fmaxf(m[j], sc[j]);
-                    const float c = exp2_fast(m[j] - m_new);
-                    l[j] *= c;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) acc[j][e] *= c;
-                    m[j] = m_new;
-                }
-            }
+        for (int j = 0; j < QG; j++) grow |= mt[j] > m[j];
+        if (__any(grow)) { // some row's maximum moves: rescale what was summed so far
 #pragma unroll
             for (int j = 0; j < QG; j++) {
-                const float p = valid ? exp2_fast(sc[j] - m[j]) : 0.f;
+                const float m_new = fmaxf(m[j], mt[j]);
+                const float c = exp2_fast(m[j] - m_new);
+                l[j] *= c;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[j][e] *= c;
+                m[j] = m_new;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < PD; u++) {
+#pragma unroll
+            for (int j = 0; j < QG; j++) {
+                const float p = valid[u] ? exp2_fast(sc[u][j] - m[j]) : 0.f;
                 l[j] += p;
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[j][e] = fmaf(p, v[e], acc[j][e]);
+                for (int e = 0; e < 8; e++) acc[j][e] = fmaf(p, v[u][e], acc[j][e]);
             }
         }
     }
