@@ -66,7 +66,15 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
     constexpr int PD = QG >= 8 ? 2 : 4; // steps in flight and per pass through the phases (4 at 8 heads: over 256 registers, one block per CU, slower)
     __shared__ float qs[QG * HS];
     __shared__ float kvnew[2][HS];
-    __shared__ float comb[NWV][QG][HS + 2];
+    // With 4 or 8 query heads per kv head the four 16-lane rows of every wave hand their partial results
+    // over through (dynamic) LDS: merging them with cross-row shuffles first takes 10 shuffles per head and
+    // step, 160 at 8 heads, a fifth of the kernel at long contexts.
+    constexpr bool kRowsInLds = QG >= 4;
+    constexpr int NR = kRowsInLds ? NWV * 4 : NWV; // partial results that meet in LDS
+    __shared__ float comb_s[kRowsInLds ? 1 : NWV][QG][HS + 2];
+    __shared__ float wts[QG][16], m_all[QG], den_all[QG];
+    extern __shared__ float comb_d[]; // [NR][QG][HS + 2] when kRowsInLds
+    float(*comb)[QG][HS + 2] = kRowsInLds ? reinterpret_cast<float(*)[QG][HS + 2]>(comb_d) : comb_s;
     const int kvh = blockIdx.x, sp = blockIdx.y;
     const int pos = A.dpos ? A.dpos[0] : A.pos;
     const int t0 = sp * A.ts;
@@ -262,49 +270,83 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
         }
     }
 
-    // merge the 4 rows of the wave (lanes 16 and 32 apart hold the same dims)
+    if constexpr (!kRowsInLds) {
+        // merge the 4 rows of the wave (lanes 16 and 32 apart hold the same dims)
 #pragma unroll
-    for (int step = 16; step <= 32; step *= 2) {
+        for (int step = 16; step <= 32; step *= 2) {
 #pragma unroll
-        for (int j = 0; j < QG; j++) {
-            const float mo = __shfl_xor(m[j], step);
-            const float lo = __shfl_xor(l[j], step);
-            const float M = fmaxf(m[j], mo);
-            const float w1 = exp2_fast(m[j] - M), w2 = exp2_fast(mo - M);
-            l[j] = l[j] * w1 + lo * w2;
+            for (int j = 0; j < QG; j++) {
+                const float mo = __shfl_xor(m[j], step);
+                const float lo = __shfl_xor(l[j], step);
+                const float M = fmaxf(m[j], mo);
+                const float w1 = exp2_fast(m[j] - M), w2 = exp2_fast(mo - M);
+                l[j] = l[j] * w1 + lo * w2;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float ao = __shfl_xor(acc[j][e], step);
-                acc[j][e] = acc[j][e] * w1 + ao * w2;
+                for (int e = 0; e < 8; e++) {
+                    const float ao = __shfl_xor(acc[j][e], step);
+                    acc[j][e] = acc[j][e] * w1 + ao * w2;
+                }
+                m[j] = M;
             }
-            m[j] = M;
         }
     }
-    if (lane < 16) {
+    if (kRowsInLds || lane < 16) {
+        const int slot = kRowsInLds ? wave * 4 + (lane >> 4) : wave;
 #pragma unroll
         for (int j = 0; j < QG; j++) {
-            *reinterpret_cast<float4 *>(&comb[wave][j][ds * 8]) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
-            *reinterpret_cast<float4 *>(&comb[wave][j][ds * 8 + 4]) =
+            *reinterpret_cast<float4 *>(&comb[slot][j][ds * 8]) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+            *reinterpret_cast<float4 *>(&comb[slot][j][ds * 8 + 4]) =
                 make_float4(acc[j][4], acc[j][5], acc[j][6], acc[j][7]);
             if (ds == 0) {
-                comb[wave][j][HS] = m[j];
-                comb[wave][j][HS + 1] = l[j];
+                comb[slot][j][HS] = m[j];
+                comb[slot][j][HS + 1] = l[j];
             }
         }
     }
     __syncthreads();
-    // merge the waves; one thread per (head, dim)
+    if constexpr (kRowsInLds) {
+        // weights of the 16 partial results of every head: one thread per (head, partial), a head per 16-lane row
+        if (tid < QG * 16) {
+            const int j = tid >> 4, e = tid & 15;
+            const float me = comb[e][j][HS];
+            float M = me;
+            M = fmaxf(M, dpp_xchg<0xB1>(M));
+            M = fmaxf(M, dpp_xchg<0x4E>(M));
+            M = fmaxf(M, dpp_xchg<0x141>(M));
+            M = fmaxf(M, dpp_xchg<0x140>(M));
+            const float w = exp2_fast(me - M);
+            float wl = w * comb[e][j][HS + 1];
+            wl += dpp_xchg<0xB1>(wl);
+            wl += dpp_xchg<0x4E>(wl);
+            wl += dpp_xchg<0x141>(wl);
+            wl += dpp_xchg<0x140>(wl);
+            wts[j][e] = w;
+            if (e == 0) {
+                m_all[j] = M;
+                den_all[j] = wl;
+            }
+        }
+        __syncthreads();
+    }
+    // merge; one thread per (head, dim)
     for (int idx = tid; idx < QG * HS; idx += NT) {
         const int j = idx >> 7, d = idx & 127;
-        float M = comb[0][j][HS];
+        float M, num = 0.f, den = 0.f;
+        if constexpr (kRowsInLds) {
 #pragma unroll
-        for (int w = 1; w < NWV; w++) M = fmaxf(M, comb[w][j][HS]);
-        float num = 0.f, den = 0.f;
+            for (int w = 0; w < NR; w++) num = fmaf(wts[j][w], comb[w][j][d], num);
+            M = m_all[j];
+            den = den_all[j];
+        } else {
+            M = comb[0][j][HS];
 #pragma unroll
-        for (int w = 0; w < NWV; w++) {
-            const float e = exp2_fast(comb[w][j][HS] - M);
-            num = fmaf(e, comb[w][j][d], num);
-            den = fmaf(e, comb[w][j][HS + 1], den);
+            for (int w = 1; w < NR; w++) M = fmaxf(M, comb[w][j][HS]);
+#pragma unroll
+            for (int w = 0; w < NR; w++) {
+                const float e = exp2_fast(comb[w][j][HS] - M);
+                num = fmaf(e, comb[w][j][d], num);
+                den = fmaf(e, comb[w][j][HS + 1], den);
+            }
         }
         const int h = kvh * QG + j;
         if (A.n_splits == 1) {
@@ -751,7 +793,16 @@ __global__ __launch_bounds__(512) void attn_combine_kernel(const AttnDecode A) {
 
 template <int QG>
 int attn_launch_qg(const AttnDecode &a, hipStream_t st) {
-    hipLaunchKernelGGL((attn_decode_kernel<QG, 4>), dim3(a.n_kv_heads, a.n_splits), dim3(256), 0, st, a);
+    constexpr size_t lds = QG >= 4 ? (size_t)16 * QG * 130 * sizeof(float) : 0; // the partial results of 16 rows
+    if (lds > 48 * 1024) {
+        static bool raised = false; // per instantiation
+        if (!raised) {
+            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_decode_kernel<QG, 4>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((attn_decode_kernel<QG, 4>), dim3(a.n_kv_heads, a.n_splits), dim3(256), lds, st, a);
     L2_HIP(hipGetLastError());
     return L2_OK;
 }
