@@ -197,52 +197,56 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
         // all weights and weighted sums — so that the dependent chains of one step (dot product, four
         // cross-lane adds, exponential) interleave with those of the others: a block is often alone on its
         // CU, one wave per SIMD, and nothing else fills the gaps between dependent instructions.
-        float v[PD][8];
+        float k[PD][8], v[PD][8];
         float sc[PD][QG];
         bool valid[PD];
         float mt[QG];
-#pragma unroll
-        for (int j = 0; j < QG; j++) mt[j] = kNoScore;
 #pragma unroll
         for (int u = 0; u < PD; u++) {
             const int t = t0 + (tile * PD + u) * TSTEP + tl;
             valid[u] = t < t1;
             const Step &d = pipe[u];
-            float k[8] = {d.k0.x, d.k0.y, d.k0.z, d.k0.w, d.k1.x, d.k1.y, d.k1.z, d.k1.w};
+            const float kk[8] = {d.k0.x, d.k0.y, d.k0.z, d.k0.w, d.k1.x, d.k1.y, d.k1.z, d.k1.w};
             const float vv[8] = {d.v0.x, d.v0.y, d.v0.z, d.v0.w, d.v1.x, d.v1.y, d.v1.z, d.v1.w};
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[u][e] = vv[e];
+            for (int e = 0; e < 8; e++) k[u][e] = kk[e], v[u][e] = vv[e];
             if (__any(t == pos)) { // once per block: the row of the new position comes from LDS, not from the cache
                 const bool is_new = t == pos;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    k[e] = is_new ? kvnew[0][ds * 8 + e] : k[e];
+                    k[u][e] = is_new ? kvnew[0][ds * 8 + e] : k[u][e];
                     v[u][e] = is_new ? kvnew[1][ds * 8 + e] : v[u][e];
                 }
             }
 #pragma unroll
             for (int e = 0; e < 8; e++) v[u][e] = valid[u] ? v[u][e] : 0.f; // a row past the end may hold anything, NaN included
+        }
 #pragma unroll
-            for (int j = 0; j < QG; j++) {
+        for (int j = 0; j < QG; j++) {
+            float qj[8];
+            if constexpr (kQInLds) { // one read of the head's q for all the steps of the tile
+                const float4 a = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8]);
+                const float4 b = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8 + 4]);
+                qj[0] = a.x, qj[1] = a.y, qj[2] = a.z, qj[3] = a.w, qj[4] = b.x, qj[5] = b.y, qj[6] = b.z, qj[7] = b.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) qj[e] = q[j][e];
+            }
+            float mj = kNoScore;
+#pragma unroll
+            for (int u = 0; u < PD; u++) {
                 float s = 0.f;
-                if constexpr (kQInLds) {
-                    const float4 a = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8]);
-                    const float4 b = *reinterpret_cast<const float4 *>(&qs[j * HS + ds * 8 + 4]);
-                    const float qj[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
-                    for (int e = 0; e < 8; e++) s = fmaf(qj[e], k[e], s);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; e++) s = fmaf(q[j][e], k[e], s);
-                }
+                for (int e = 0; e < 8; e++) s = fmaf(qj[e], k[u][e], s);
                 s += dpp_xchg<0xB1>(s);
                 s += dpp_xchg<0x4E>(s);
                 s += dpp_xchg<0x141>(s);
                 s += dpp_xchg<0x140>(s);
                 s = valid[u] ? s * scale : kNoScore;
                 sc[u][j] = s;
-                mt[j] = fmaxf(mt[j], s);
+                mj = fmaxf(mj, s);
             }
+            mt[j] = mj;
         }
         bool grow = false;
 #pragma unroll
