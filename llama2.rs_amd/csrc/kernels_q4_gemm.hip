@@ -98,19 +98,25 @@ __device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
     return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_offset);
 }
 
-// Software pipeline of the K loop.  Everything a K step needs is loaded PW (weights, zeros, scales) or
-// XP (the activation tile) steps ahead, unconditionally (steps past the end of the block's K slice
-// re-read its last step), into rings of registers indexed statically by the position in the loop body,
-// which is unrolled PW times.  Loads return in order, so a wait for the oldest ring slot leaves all the
-// younger ones in flight; with one block of 4 waves on a CU this depth, not occupancy, hides HBM latency.
+// Software pipeline of the K loop.  The weights of a K step are loaded WR steps ahead, its activation
+// tile XP steps ahead, the scales and zero points of PW groups once per PW steps, all unconditionally
+// (steps past the end of the block's K slice re-read its last step), into rings of registers indexed
+// statically by the position in the loop body, which is unrolled PW times.  Loads return in order, so a
+// wait for the oldest ring slot leaves the younger ones in flight; within a step the activation tile is
+// requested before the weights, because the end of the step waits for it (it comes from the L2) and would
+// otherwise wait for the weights requested before it as well.  Shallow rings on purpose: at K steps of 128,
+// depths of 4 and 2 instead of 2 and 1 cost 34 more registers and were 3 % slower.
 constexpr int kGemmPW = 4;
-constexpr int kGemmXP = 2;
+// ring depths in K steps: 256 k ahead for the weights, 128 k for the activation tile
+constexpr int gemm_wr(int kstep) { return 256 / kstep; }
+constexpr int gemm_xp(int kstep) { return 128 / kstep; }
 
 template <int G, int NB, int KSTEP>
 __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
                                                       float *__restrict__ ws, int KS, int partials) {
     Q4G_STAMP(0);
-    constexpr int PW = kGemmPW, XP = kGemmXP;
+    constexpr int PW = kGemmPW, XP = gemm_xp(KSTEP), WR = gemm_wr(KSTEP);
+    static_assert(PW % WR == 0 && PW % XP == 0, "ring slots are indexed by the position in the unrolled body");
     constexpr int W = KSTEP / 64;        // sub-steps of 64 k per K step
     constexpr int kXRow = KSTEP + kXPad; // halves per staged token row
     static_assert(KSTEP == 64 || G >= KSTEP, "a longer K step stays inside one group");
@@ -231,14 +237,14 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     };
 
     XStage xr[XP];
-    WStage wr[PW];
+    WStage wr[WR];
     float2 gs2 = make_float2(0.f, 0.f);
     int32_t zs2 = 0;
     if constexpr (SA) gs2 = fetch_gs(0), zs2 = fetch_zs(0);
 #pragma unroll
     for (int j = 0; j < XP; j++) fetch_x(kit0 + j, xr[j]);
 #pragma unroll
-    for (int j = 0; j < PW; j++) fetch_w(kit0 + j, wr[j]);
+    for (int j = 0; j < WR; j++) fetch_w(kit0 + j, wr[j]);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the loop's waits then reflect its own order only
     store_x(0, xr[0]);
     if constexpr (SA) store_gs(0, gs2), store_zs(0, zs2);
@@ -252,7 +258,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             const int kit = kit0 + stepi;
             const int buf = u & 1; // PW is even: the parity of the step
             // this step's weights -> registers of their own, then refill the slot
-            const int zword = SA ? zsc[(stepi / PW) & 1][u][(wave * 32 + r) >> 3] : wr[u].z;
+            const int zword = SA ? zsc[(stepi / PW) & 1][u][(wave * 32 + r) >> 3] : wr[u % WR].z;
             const int zn = (zword >> (4 * (orow & 7))) & 15;
             DequantConsts dc;
             dc.mask_lo = 0x000F000Fu, dc.mask_hi = 0x00F000F0u, dc.magic = 0x64006400u;
@@ -261,12 +267,12 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             dc.neg_off = h2{off, off};
             dc.neg_off16 = h2{off16, off16};
             dc.sixteenth = h2{(_Float16)0.0625f, (_Float16)0.0625f};
-            const _Float16 s1 = (_Float16)wr[u].s;
+            const _Float16 s1 = (_Float16)wr[u % WR].s;
             const h2 s16 = h2{s1, s1};
             uint32_t wd[W][4];
 #pragma unroll
             for (int sw = 0; sw < W; sw++) {
-                wd[sw][0] = wr[u].w[sw].x, wd[sw][1] = wr[u].w[sw].y, wd[sw][2] = wr[u].w[sw].z, wd[sw][3] = wr[u].w[sw].w;
+                wd[sw][0] = wr[u % WR].w[sw].x, wd[sw][1] = wr[u % WR].w[sw].y, wd[sw][2] = wr[u % WR].w[sw].z, wd[sw][3] = wr[u % WR].w[sw].w;
                 asm volatile("" : "+v"(wd[sw][0]), "+v"(wd[sw][1]), "+v"(wd[sw][2]), "+v"(wd[sw][3])::"memory");
             }
             // The ring slot stays in its own registers up to here (the copies above live elsewhere), so the
@@ -274,27 +280,28 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
             // fresh ones and is copied back at the loop's end, behind a wait for the load just issued.
 #pragma unroll
             for (int sw = 0; sw < W; sw++)
-                asm volatile("" : "+v"(wr[u].w[sw].x), "+v"(wr[u].w[sw].y), "+v"(wr[u].w[sw].z), "+v"(wr[u].w[sw].w));
-            if constexpr (!SA) asm volatile("" : "+v"(wr[u].z));
+                asm volatile("" : "+v"(wr[u % WR].w[sw].x), "+v"(wr[u % WR].w[sw].y), "+v"(wr[u % WR].w[sw].z), "+v"(wr[u % WR].w[sw].w));
+            if constexpr (!SA) asm volatile("" : "+v"(wr[u % WR].z));
             __builtin_amdgcn_sched_barrier(0);
             // The refills of this step (ring slot u of the weights, slot u % XP of the activations, once per
             // round the next PW groups' scales and zero points) are issued one at a time between the MFMA
             // steps below: a global load takes the wave hundreds of cycles to issue when the address unit is
             // busy, and issued in one burst here those cycles stood in front of the first MFMA.
-            const int kc_w = min(kit + PW, kit1 - 1);
+            const int kc_w = min(kit + WR, kit1 - 1);
             const uint32_t kb_x = (uint32_t)min(kit + XP, kit1 - 1) * (uint32_t)(KSTEP * 2);
             constexpr int NL = W + 1 + PIECES + 1;
             auto refill = [&](const int i) __attribute__((always_inline)) {
-                if (i < W) {
-                    wr[u].w[i] = ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc_w * (2 * W) + 2 * i + h) << 4);
-                } else if (i == W) {
+                if (i < PIECES) { // the activations first: the end of the step waits for them, not for what follows
+                    xr[u % XP].v[i] = ld_at<uint4>(xh, xoff[i] + kb_x);
+                } else if (i < PIECES + W) {
+                    wr[u % WR].w[i - PIECES] =
+                        ld_at<uint4>(qw_base, (uint32_t)(orow * C4 + kc_w * (2 * W) + 2 * (i - PIECES) + h) << 4);
+                } else if (i == PIECES + W) {
                     if constexpr (!SA) {
                         const int g = (kc_w * KSTEP + 32 * h) / G;
-                        wr[u].z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
-                        wr[u].s = ld_at<float>(sc_base, (uint32_t)(orow * groups + g) << 2);
+                        wr[u % WR].z = ld_at<int32_t>(qz_base, (uint32_t)((orow >> 3) * groups + g) << 2);
+                        wr[u % WR].s = ld_at<float>(sc_base, (uint32_t)(orow * groups + g) << 2);
                     }
-                } else if (i < W + 1 + PIECES) {
-                    xr[u % XP].v[i - W - 1] = ld_at<uint4>(xh, xoff[i - W - 1] + kb_x);
                 } else if (SA && u == 0) {
                     gs2 = fetch_gs(base / PW + 1), zs2 = fetch_zs(base / PW + 1);
                 }
