@@ -138,9 +138,12 @@ TINY_GQA = ck.Dims(dim=512, hidden_dim=768, n_layers=2, n_heads=4, n_kv_heads=2,
                    seq_len=80, group_size=128)
 MID = ck.Dims(dim=1024, hidden_dim=2816, n_layers=3, n_heads=8, n_kv_heads=2, vocab_size=2000,
               seq_len=256, group_size=32)
+# rows of 3 waves (144 chunks, the last wave ragged) behind an rmsnorm, as q|k|v and w1|w3 of the 13B preset
+WIDE = ck.Dims(dim=4608, hidden_dim=1536, n_layers=2, n_heads=36, n_kv_heads=9, vocab_size=300,
+               seq_len=64, group_size=128)
 
 
-@pytest.mark.parametrize("dims", [TINY, TINY_GQA, MID], ids=["mha_g64", "gqa_g128", "gqa_g32"])
+@pytest.mark.parametrize("dims", [TINY, TINY_GQA, MID, WIDE], ids=["mha_g64", "gqa_g128", "gqa_g32", "wide_g128"])
 def test_forward_logits_and_cache_vs_oracle(ops, oracle, dims, tmp_path):
     img = ck.synth_weights_image(dims, seed=11)
     path = str(tmp_path / "m.bin")
