@@ -317,36 +317,64 @@ struct l2_model {
     std::vector<ProfRec> prof;
 };
 
+
 enum { K_EMBED = 0, K_Q4_QKV, K_ROPE_KV, K_ATTENTION, K_Q4_WO, K_Q4_W13, K_Q4_W2, K_CLASSIFIER, K_NEXT_TOKEN,
        K_NCLASS };
 static const char *const kClassNames[K_NCLASS] = {"embed", "q4_qkv", "rope_kv", "attention", "q4_wo",
                                                   "q4_w13", "q4_w2", "classifier", "next_token"};
 static constexpr int kMaxSplits = 64;
 
-// Time one launch (profiling runs only).  The q4 launches hand their events to
-// the dispatch itself; the others are bracketed by event records on the stream.
-#define LAUNCH(cls_, call)                                                          \
-    do {                                                                            \
-        if (m->prof_on) {                                                           \
-            l2_model::ProfRec r_{cls_, nullptr, nullptr};                           \
-            L2_HIP(hipEventCreate(&r_.e0));                                         \
-            L2_HIP(hipEventCreate(&r_.e1));                                         \
-            const bool q4_ = m->d.group_size != 0 && ((cls_) == K_Q4_QKV || (cls_) == K_Q4_WO || (cls_) == K_Q4_W13 || (cls_) == K_Q4_W2); \
-            if (q4_) {                                                              \
-                g_q4_prof.start = r_.e0;                                            \
-                g_q4_prof.stop = r_.e1;                                             \
-                g_q4_prof.armed = true;                                             \
-                L2_TRY(call);                                                       \
-                g_q4_prof.armed = false;                                            \
-            } else {                                                                \
-                L2_HIP(hipEventRecord(r_.e0, m->stream));                           \
-                L2_TRY(call);                                                       \
-                L2_HIP(hipEventRecord(r_.e1, m->stream));                           \
-            }                                                                       \
-            m->prof.push_back(r_);                                                  \
-        } else {                                                                    \
-            L2_TRY(call);                                                           \
-        }                                                                           \
+// Time one launch (profiling runs only).  The q4 launches of the streaming form hand their events to the
+// dispatch itself; everything else is bracketed by event records on the stream.  Events of a launch that
+// failed, or that nobody recorded, are destroyed here and leave no record.
+template <class F>
+static int timed_launch(l2_model *m, int cls, F &&launch) {
+    static const bool tile_form = []() {
+        const char *v = getenv("L2_Q4_IMPL");
+        return v && !strcmp(v, "tile");
+    }();
+    l2_model::ProfRec r{cls, nullptr, nullptr};
+    auto drop = [&]() {
+        if (r.e0) (void)hipEventDestroy(r.e0);
+        if (r.e1) (void)hipEventDestroy(r.e1);
+    };
+    hipError_t e = hipEventCreate(&r.e0);
+    if (e == hipSuccess) e = hipEventCreate(&r.e1);
+    if (e != hipSuccess) {
+        drop();
+        return l2_fail(L2_ERR_HIP, "hipEventCreate: %s", hipGetErrorString(e));
+    }
+    const bool q4 = !tile_form && m->d.group_size != 0 &&
+                    (cls == K_Q4_QKV || cls == K_Q4_WO || cls == K_Q4_W13 || cls == K_Q4_W2);
+    int rc = L2_OK;
+    bool recorded = true;
+    if (q4) {
+        g_q4_prof.start = r.e0;
+        g_q4_prof.stop = r.e1;
+        g_q4_prof.armed = true;
+        rc = launch();
+        recorded = !g_q4_prof.armed; // a form of the kernel that does not take the events leaves them armed
+        g_q4_prof.armed = false;
+    } else {
+        e = hipEventRecord(r.e0, m->stream);
+        if (e == hipSuccess) rc = launch();
+        if (e == hipSuccess && rc == L2_OK) e = hipEventRecord(r.e1, m->stream);
+        if (e != hipSuccess && rc == L2_OK) rc = l2_fail(L2_ERR_HIP, "hipEventRecord: %s", hipGetErrorString(e));
+    }
+    if (rc != L2_OK || !recorded) {
+        drop();
+        return rc;
+    }
+    m->prof.push_back(r);
+    return L2_OK;
+}
+
+#define LAUNCH(cls_, call)                                                   \
+    do {                                                                     \
+        if (m->prof_on)                                                      \
+            L2_TRY(timed_launch(m, (cls_), [&]() -> int { return (call); })); \
+        else                                                                 \
+            L2_TRY(call);                                                    \
     } while (0)
 
 struct StepGraph {
@@ -1018,7 +1046,16 @@ static void attn_split_policy(int n_t, int n_kv_heads, int *ts_out, int *n_split
 // in the input order (g_index) of whoever reads it next.
 static int forward_enqueue_dense(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits);
 
+static int check_position(const l2_model *m, int max_pos) {
+    // No kernel clamps a position: the RoPE table and the cache end at max_seq (the reference panics on its
+    // fixed [SEQ_LEN] arrays, src/models.rs:29-33).
+    if (max_pos < 0 || max_pos >= m->max_seq)
+        return l2_fail(L2_ERR_RANGE, "position %d outside 0..%d", max_pos, m->max_seq - 1);
+    return L2_OK;
+}
+
 static int forward_enqueue(l2_model *m, l2_state *s, int B, int max_pos, bool want_logits) {
+    L2_TRY(check_position(m, max_pos));
     if (m->d.group_size == 0) return forward_enqueue_dense(m, s, B, max_pos, want_logits);
     const l2_dims &d = m->d;
     const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
@@ -1200,6 +1237,7 @@ static int ensure_batch_mfma(l2_model *m, int B) {
 // element-wise steps as kernels of their own.  Logits are never produced here
 // (src/models.rs:288).
 static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
+    L2_TRY(check_position(m, max_pos));
     const l2_dims &d = m->d;
     const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
     hipStream_t st = m->stream;
@@ -1433,12 +1471,26 @@ static int loop_begin(l2_model *m, int n_prompt, int pos0) {
     return set_i32_launch(m->dloop, n_prompt, m->dloop + 1, pos0, m->stream);
 }
 
+// Position at which prefill<64>, <32>, ... <2> (src/inference.rs:78-127) leave off for a prompt of n_prompt
+// tokens: each takes chunks of A positions while pos + A < n_prompt (:24).
+int l2_prefill_ladder_end(int n_prompt) {
+    int pos = 0;
+    for (int A = 64; A >= 2; A /= 2)
+        while (pos + A < n_prompt) pos += A;
+    return pos;
+}
+
 extern "C" int l2_generate_greedy(l2_model *m, l2_state *s, const int32_t *prompt, int n_prompt, int steps,
                                   int use_prefill, int32_t *out_ids, int *n_out, double *ms) {
     if (!m || !s || !out_ids || !n_out || (n_prompt > 0 && !prompt)) return l2_fail(L2_ERR_ARG, "null argument");
     if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
     if (n_prompt < 0 || steps < 0) return l2_fail(L2_ERR_ARG, "negative count");
     if (steps > m->max_seq) return l2_fail(L2_ERR_RANGE, "steps %d exceeds the cache length %d", steps, m->max_seq);
+    // The ladder runs whatever `steps` is: a prompt it would carry past the cache is refused before any launch
+    // (the reference panics there on its fixed [SEQ_LEN] arrays).
+    if (use_prefill && l2_prefill_ladder_end(n_prompt) > m->max_seq)
+        return l2_fail(L2_ERR_RANGE, "a prompt of %d tokens prefills %d positions, the cache holds %d", n_prompt,
+                       l2_prefill_ladder_end(n_prompt), m->max_seq);
     for (int i = 0; i < n_prompt; i++)
         if (prompt[i] < 0 || prompt[i] >= m->d.vocab_size)
             return l2_fail(L2_ERR_RANGE, "prompt token %d outside 0..%d", prompt[i], m->d.vocab_size - 1);

@@ -82,17 +82,6 @@ __device__ __forceinline__ h8 dequant8(uint32_t w, const DequantConsts &c, h2 sc
     return a.v;
 }
 
-#if defined(Q4G_TS) // measurement build only: per-block timestamps (100 MHz counter)
-__device__ unsigned long long q4g_ts[4096 * 4];
-#define Q4G_STAMP(k)                                                                                    \
-    do {                                                                                                \
-        const unsigned bid_ = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);          \
-        if (threadIdx.x == 0 && bid_ < 4096) q4g_ts[bid_ * 4 + (k)] = wall_clock64();                  \
-    } while (0)
-#else
-#define Q4G_STAMP(k)
-#endif
-
 template <class T>
 __device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
     return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_offset);
@@ -114,7 +103,6 @@ constexpr int gemm_xp(int kstep) { return 128 / kstep; }
 template <int G, int NB, int KSTEP>
 __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
                                                       float *__restrict__ ws, int KS, int partials) {
-    Q4G_STAMP(0);
     constexpr int PW = kGemmPW, XP = gemm_xp(KSTEP), WR = gemm_wr(KSTEP);
     static_assert(PW % WR == 0 && PW % XP == 0, "ring slots are indexed by the position in the unrolled body");
     constexpr int W = KSTEP / 64;        // sub-steps of 64 k per K step
@@ -249,7 +237,6 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     store_x(0, xr[0]);
     if constexpr (SA) store_gs(0, gs2), store_zs(0, zs2);
     __syncthreads();
-    Q4G_STAMP(1);
 
     // One K step; u = step % PW indexes the register rings (a compile-time constant where it is called).
     auto k_step = [&](const int stepi, const int u) __attribute__((always_inline)) {
@@ -369,7 +356,6 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     for (int u = 0; u < PW - 1; u++)
         if (u < n_rem) k_step(n_full * PW + u, u);
 
-    Q4G_STAMP(2);
     // C layout: lane (col n = l%32 -> token, h = l/32), register i -> row (i/4)*8 + h*4 + i%4.
     // Stored as it stands, every store instruction would touch 64 separate 16-byte pieces; instead each
     // wave turns its 32 rows x 32 tokens through LDS (the activation buffers are free now) so that a
@@ -417,16 +403,7 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                 for (int e = 0; e < 4; e++) E.sc_out[c][row + E.sc_idx[c][o + e]] = vals[e];
         }
     }
-    Q4G_STAMP(3);
 }
-
-#if defined(Q4G_TS)
-} // namespace
-extern "C" int l2_debug_gemm_ts(unsigned long long *out, int n) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(q4g_ts), (size_t)n * 8);
-}
-namespace {
-#endif
 
 // Adds the KS partial tiles of a split-K GEMM in slice order and runs the epilogue; a thread owns four
 // consecutive outputs of one token (every `out` is a multiple of 32).

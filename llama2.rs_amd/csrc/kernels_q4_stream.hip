@@ -15,18 +15,16 @@
 // barrier per tile of P*S rows, one thread per row adds them in a fixed order
 // and runs the epilogue.  No atomics: results are bit-stable.
 //
-// Integer form (IDOT).  The vector ALU is the co-bottleneck of the fp32 form
-// (one FMA, one convert-equivalent and 3/8 of a mask per nibble), so the default
-// form keeps the arithmetic in integers: after staging, the block quantises x
-// once, chunk by chunk, to 24-bit fixed point against a power-of-two step
-// (delta = 2^(e-22), |x| < 2^e within the chunk) and stores it as six planes of
-// balanced base-16 digits (-8..7), 8 digits per word in the nibble order of the
-// weights.  A weight word XOR 0x88888888 is the 8 signed nibbles n - 8, so
-// v_dot8_i32_i4 multiplies one weight word with one digit word: 24 instructions
-// per 32 weights instead of ~76, exact integer sums, and
+// Integer form (MODE 1, selected with L2_Q4_IMPL=idot; the fp32 form is the default).  The vector ALU is
+// the co-bottleneck of the fp32 form (one FMA, one convert-equivalent and 3/8 of a mask per nibble).  The
+// integer form quantises x once per block after staging, chunk by chunk, to 24-bit fixed point against a
+// power-of-two step (delta = 2^(e-22), |x| < 2^e within the chunk) and stores it as six planes of balanced
+// base-16 digits (-8..7), 8 digits per word in the nibble order of the weights.  A weight word XOR 0x88888888
+// is the 8 signed nibbles n - 8, so v_dot8_i32_i4 multiplies one weight word with one digit word: 24
+// instructions per 32 weights instead of ~76, exact integer sums, and
 //   sum_k (n_k - z1) x_k = delta * (I - (z1 - 8) * sum_k q_k),  I = sum_d 16^d a_d.
-// The quantisation error (2^-23 of the chunk maximum per element) is of the
-// size of fp32 rounding.
+// The quantisation error (2^-23 of the chunk maximum per element) is of the size of fp32 rounding.  Its
+// quantisation prologue costs more than the shorter loop saves on the shapes measured, hence not the default.
 #include <string.h>
 
 #include "q4_common.h"
@@ -131,16 +129,6 @@ __device__ __forceinline__ void st_at(float *base, uint32_t byte_offset, float v
     *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + byte_offset) = v;
 }
 
-#if defined(Q4S_TS) // measurement build only: per-block timestamps (100 MHz counter)
-__device__ unsigned long long q4s_ts[1024 * 8];
-#define Q4S_STAMP(k)                                                                  \
-    do {                                                                              \
-        if (threadIdx.x == 0 && blockIdx.x < 1024) q4s_ts[blockIdx.x * 8 + (k)] = wall_clock64(); \
-    } while (0)
-#else
-#define Q4S_STAMP(k)
-#endif
-
 struct RowData {
     uint4 w;
     float s;
@@ -165,7 +153,6 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     __shared__ float red[NW];
     __shared__ float part[2][TR][NM][PW];
 
-    Q4S_STAMP(0);
     const int in = L.in;
     const int C = in >> 5;
     const int xstride = C * kChunkPad + C;
@@ -236,12 +223,10 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
             stage_issue<NW>(L.m[mi + q].x + (size_t)b * in, L.m[mi + q].wn, in, 0, tid, xr[q]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    Q4S_STAMP(6);
     RowData pipe[P][NM];
 #pragma unroll
     for (int u = 0; u < P; u++) fetch(u, pipe[u]);
     __builtin_amdgcn_sched_barrier(0);
-    Q4S_STAMP(7);
 
     // this lane's slice of x, for good: 32 floats, or 24 digit words + step + sum of q
     float x[NM][IDOT ? 1 : 32];
@@ -273,7 +258,6 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         }
         sx[0] = t;
         xdelta[0] = 0.f;
-        Q4S_STAMP(1);
     } else {
         // stage x for the whole block, then take this lane's chunk into registers
         float ssq = 0.f;
@@ -285,7 +269,6 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
             p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
             if (q == 0) ssq = p;
         }
-        Q4S_STAMP(1);
         if (norm) {
             ssq = wave_sum(ssq);
             if (lane == 0) red[wave] = ssq;
@@ -356,9 +339,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     // was staged). The compiler's wait counts inside the loop are then those of
     // the steady state alone: vmcnt leaves the P - 1 younger rows in flight.
     // Otherwise the issue order of the prologue leaks into the loop's waits.
-    Q4S_STAMP(2);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0), expcnt and lgkmcnt untouched
-    Q4S_STAMP(3);
     // Epilogue operands, uniform for the block.
     const Q4Epi &E = L.e;
     const int epi_kind = E.kind;
@@ -459,7 +440,6 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         __syncthreads();
         if (epi) tile_finish(eo, res_v, sidx);
         buf ^= 1;
-        Q4S_STAMP(4);
     }
     if (n_rem > 0) { // the rows already in the pipe: no refill, nothing younger to leave in flight
         const int eo = row0 + n_full * TR + tid;
@@ -482,16 +462,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         __syncthreads();
         if (epi) tile_finish(eo, res_v, sidx);
     }
-    Q4S_STAMP(5);
 }
-
-#if defined(Q4S_TS)
-} // namespace
-extern "C" int l2_debug_q4_ts(unsigned long long *out, int n) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(q4s_ts), (size_t)n * 8);
-}
-namespace {
-#endif
 
 // Rows per block for a block of NW waves and tiles of TR rows: a whole number of rounds over the CUs, as
 // many blocks per CU as 16 waves and the LDS allow; every block gets the same number of rows; several

@@ -42,6 +42,9 @@ int l2_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3))
         if (rc_ != L2_OK) return rc_; \
     } while (0)
 
+// Position at which the prefill ladder 64/32/16/8/4/2 (src/inference.rs:78-127) leaves off.
+int l2_prefill_ladder_end(int n_prompt);
+
 // ---- device views ---------------------------------------------------------
 
 // One QLinear resident in device memory, `.bin` layout (src/gptq.rs:68-84),

@@ -196,6 +196,34 @@ static const char *token_text(const l2_tokenizer *t, int token, int next, int *l
     return s.data();
 }
 
+// char::is_whitespace (the White_Space property), which str::trim uses (src/inference.rs:63)
+static bool is_unicode_space(uint32_t c) {
+    return (c >= 0x09 && c <= 0x0D) || c == 0x20 || c == 0x85 || c == 0xA0 || c == 0x1680 ||
+           (c >= 0x2000 && c <= 0x200A) || c == 0x2028 || c == 0x2029 || c == 0x202F || c == 0x205F || c == 0x3000;
+}
+
+// The code point that starts at byte i of valid UTF-8, and its length in bytes.
+static uint32_t utf8_at(const std::string &s, size_t i, size_t *len) {
+    const unsigned char c = (unsigned char)s[i];
+    const size_t k = c < 0x80 ? 1 : (c >> 5) == 6 ? 2 : (c >> 4) == 14 ? 3 : 4;
+    uint32_t cp = k == 1 ? c : (uint32_t)(c & (0xFFu >> (k + 1)));
+    for (size_t j = 1; j < k; j++) cp = (cp << 6) | ((unsigned char)s[i + j] & 0x3Fu);
+    *len = k;
+    return cp;
+}
+
+static std::string trim_unicode(const std::string &p) {
+    size_t a = 0, b = p.size(), k;
+    while (a < b && is_unicode_space(utf8_at(p, a, &k))) a += k;
+    while (b > a) {
+        size_t q = b - 1; // start of the last character
+        while (q > a && ((unsigned char)p[q] >> 6) == 2) q--;
+        if (!is_unicode_space(utf8_at(p, q, &k))) break;
+        b = q;
+    }
+    return p.substr(a, b - a);
+}
+
 extern "C" int l2_generate(l2_model *m, l2_state *s, const l2_tokenizer *t, const char *prompt, int steps,
                            l2_random *rng, float temperature, int print_tokens, char *out, size_t out_cap,
                            int *n_tokens, int64_t *ms) {
@@ -207,53 +235,82 @@ extern "C" int l2_generate(l2_model *m, l2_state *s, const l2_tokenizer *t, cons
     // prompt: " " + trim (src/inference.rs:62-67)
     std::vector<int> prompt_tokens;
     {
-        std::string p(prompt);
-        size_t a = 0, b = p.size();
-        auto ws = [](unsigned char c) { return c == ' ' || (c >= 9 && c <= 13); };
-        while (a < b && ws((unsigned char)p[a])) a++;
-        while (b > a && ws((unsigned char)p[b - 1])) b--;
-        if (!p.empty()) L2_TRY(bpe_encode(t, " " + p.substr(a, b - a), prompt_tokens));
+        const std::string p(prompt);
+        if (!valid_utf8(p)) return l2_fail(L2_ERR_ARG, "prompt is not UTF-8");
+        if (!p.empty()) L2_TRY(bpe_encode(t, " " + trim_unicode(p), prompt_tokens));
     }
     const int n_prompt = (int)prompt_tokens.size();
-    std::vector<int32_t> prompt32(prompt_tokens.begin(), prompt_tokens.end());
+    const std::vector<int32_t> prompt32(prompt_tokens.begin(), prompt_tokens.end());
     std::vector<int32_t> ids((size_t)(steps > 0 ? steps : 1));
+    const bool prefill = l2_prefill_supported(m) != 0;
+    size_t used = 0;
+    // one token string of get_token (src/util.rs:116-123): printed at once (print_token flushes, :125-128),
+    // and, for the strings the reference returns, appended to `out`
+    auto emit = [&](int token, int next, bool returned) -> int {
+        int len;
+        const char *str = token_text(t, token, next, &len);
+        if (print_tokens) {
+            fwrite(str, 1, (size_t)len, stdout);
+            fflush(stdout);
+        }
+        if (!returned) return L2_OK;
+        if (out) {
+            if (used + (size_t)len + 1 > out_cap) return l2_fail(L2_ERR_ARG, "output buffer of %zu bytes is too small", out_cap);
+            memcpy(out + used, str, (size_t)len);
+            out[used + len] = '\0';
+        }
+        used += (size_t)len + 1;
+        return L2_OK;
+    };
     int n = 0;
-    int first_pos = 0; // position the loop starts at (the prefill ladder consumes some silently)
     const auto t0 = std::chrono::system_clock::now(); // time_in_ms, :72
-    if (temperature == 0.0f) {
+    if (temperature == 0.0f && !print_tokens) {
+        // nothing is wanted before the end: the whole loop stays on the device
         double ms_loop = 0;
-        L2_TRY(l2_generate_greedy(m, s, prompt32.data(), n_prompt, steps, l2_prefill_supported(m), ids.data(), &n, &ms_loop));
-        first_pos = steps - n;
+        L2_TRY(l2_generate_greedy(m, s, prompt32.data(), n_prompt, steps, prefill, ids.data(), &n, &ms_loop));
+        const int first_pos = prefill ? l2_prefill_ladder_end(n_prompt) : 0; // the ladder may pass `steps`
+        int token = first_pos == 0 ? 1 : prompt32[first_pos - 1];
+        for (int i = 0; i < n; i++) {
+            L2_TRY(emit(token, ids[i], true));
+            token = ids[i];
+        }
     } else {
-        // the same loop with the sampler on the host (:141-190); prefill as above
+        // the loop on the host, a token at a time, so that every string is printed when it exists and the
+        // sampler sees the logits (:141-190)
         L2_TRY(l2_state_reset(s));
         int pos = 0;
-        if (l2_prefill_supported(m)) {
-            static const int ladder[6] = {64, 32, 16, 8, 4, 2};
+        if (prefill) { // :16-44, :78-127
             std::vector<int32_t> toks(64), poss(64);
-            for (int A : ladder)
+            for (int A = 64; A >= 2; A /= 2)
                 while (pos + A < n_prompt) {
                     for (int i = 0; i < A; i++) {
                         toks[i] = pos == 0 ? 1 : prompt32[pos - 1];
                         poss[i] = pos++;
+                        L2_TRY(emit(toks[i], toks[i], false)); // :37-40
                     }
                     L2_TRY(l2_forward(m, s, toks.data(), poss.data(), A, nullptr));
                 }
         }
-        first_pos = pos;
         int32_t token = pos == 0 ? 1 : prompt32[pos - 1];
-        std::vector<float> logits((size_t)d.vocab_size);
+        L2_TRY(emit(token, token, false)); // :134-137
+        std::vector<float> logits(temperature != 0.0f ? (size_t)d.vocab_size : 0);
         while (pos < steps) {
             const int32_t p32 = pos;
-            L2_TRY(l2_forward(m, s, &token, &p32, 1, logits.data()));
-            int next;
-            if (pos < n_prompt) {
-                next = prompt32[pos];
+            int32_t next = 0;
+            if (temperature == 0.0f) {
+                L2_TRY(l2_decode_greedy(m, s, token, p32, &next)); // :160-162, argmax on the device
+                if (pos < n_prompt) next = prompt32[pos];
             } else {
-                for (int q = 0; q < d.vocab_size; q++) logits[q] /= temperature; // :166-168
-                softmax_host(logits.data(), d.vocab_size);
-                next = l2_random_sample(rng, logits.data(), d.vocab_size);
+                L2_TRY(l2_forward(m, s, &token, &p32, 1, logits.data()));
+                if (pos < n_prompt) {
+                    next = prompt32[pos];
+                } else {
+                    for (int q = 0; q < d.vocab_size; q++) logits[q] /= temperature; // :166-168
+                    softmax_host(logits.data(), d.vocab_size);
+                    next = l2_random_sample(rng, logits.data(), d.vocab_size);
+                }
             }
+            L2_TRY(emit(token, next, true)); // :178-182
             ids[n++] = next;
             token = next;
             pos++;
@@ -261,29 +318,6 @@ extern "C" int l2_generate(l2_model *m, l2_state *s, const l2_tokenizer *t, cons
     }
     const auto t1 = std::chrono::system_clock::now();
     *ms = std::chrono::duration_cast<std::chrono::milliseconds>(t1 - t0).count();
-    // token strings (:178-182), NUL separated
-    size_t used = 0;
-    int token = first_pos == 0 ? 1 : prompt32[first_pos - 1];
-    if (print_tokens) { // :134-137
-        int len;
-        const char *str = token_text(t, token, token, &len);
-        fwrite(str, 1, (size_t)len, stdout);
-    }
-    for (int i = 0; i < n; i++) {
-        int len;
-        const char *str = token_text(t, token, ids[i], &len);
-        if (print_tokens) {
-            fwrite(str, 1, (size_t)len, stdout);
-            fflush(stdout);
-        }
-        if (out) {
-            if (used + (size_t)len + 1 > out_cap) return l2_fail(L2_ERR_ARG, "output buffer of %zu bytes is too small", out_cap);
-            memcpy(out + used, str, (size_t)len);
-            out[used + len] = '\0';
-        }
-        used += (size_t)len + 1;
-        token = ids[i];
-    }
     *n_tokens = n;
     return L2_OK;
 }

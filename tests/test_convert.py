@@ -102,3 +102,30 @@ def test_converter_rejects_what_the_format_cannot_hold(tmp_path):
     (tmp_path / "quantize_config.json").write_text(json.dumps({"bits": 4, "group_size": 128}))
     with pytest.raises(ValueError):   # shapes no longer fit the declared group size
         cv.convert(str(tmp_path), str(tmp_path / "m.bin"), log=lambda s: None)
+
+
+@pytest.mark.gpu
+def test_converted_file_through_the_hip_loader(tmp_path, oracle):
+    """convert() -> l2_model_open -> transformer<1> on the GPU: the logits and the greedy tokens of the
+    converted file equal the oracle's on the same file."""
+    from llama2_rs import ops
+    dims = ck.Dims(dim=512, hidden_dim=768, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=200, seq_len=48,
+                   group_size=128)
+    _make_checkpoint(tmp_path, dims, seed=3)
+    out = str(tmp_path / "m.bin")
+    assert cv.convert(str(tmp_path), out, max_vocab_size=dims.vocab_size, max_seq_len=dims.seq_len,
+                      log=lambda s: None) == dims
+    img = np.fromfile(out, dtype=np.uint8)[ck.HEADER_BYTES:]
+    m = ops.Model(out, dims)
+    o = oracle.Model(img, dims)
+    o.new_state()
+    for pos, tk in enumerate([1, 7, 42, 5, 199]):
+        want = o.transformer([tk], [pos])
+        got = m.forward([tk], [pos])
+        scale = np.maximum(np.abs(want), np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        assert np.max(np.abs(got - want) / scale) < 1e-4, pos
+    prompt = np.array([3, 150, 9, 77, 12], np.int32)
+    got, _ = m.generate_greedy(prompt, 30, use_prefill=True)
+    np.testing.assert_array_equal(got, o.generate_greedy(prompt, 30, use_prefill=True))
+    m.close()
+    o.close()

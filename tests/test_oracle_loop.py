@@ -14,41 +14,66 @@ TINY_GQA = ck.Dims(dim=512, hidden_dim=768, n_layers=2, n_heads=4, n_kv_heads=2,
                    seq_len=80, group_size=128)
 
 
-def _split_image(img, d):
-    """Walk the image in struct order and return fp64 dense weights (independent of oracle.c)."""
+def _split_image(img, d, layers=None, names=None, max_rows=None):
+    """Walk the image in struct order and return fp64 dense weights (independent of oracle.c).
+    With `layers` / `names` only those layers of those tensors are dequantised (big models); the rest is None.
+    With `max_rows` a quantised projection of more than 2 * max_rows outputs gives its first and last max_rows
+    rows only; w["rows"][name] holds the row numbers."""
     off = [0]
+    rows_of = {}
 
-    def take(n, dt):
-        a = img[off[0]:off[0] + n * 4].view(dt)
+    def take(n, dt, want=True):
+        a = img[off[0]:off[0] + n * 4].view(dt) if want else None
         off[0] += n * 4
         return a
 
-    def qlin(n_in, n_out):
+    def wanted(name):
+        return names is None or name in names
+
+    def qlin(name, n_in, n_out):
         out = []
         g = ck.groups_of(n_in, d.group_size) if d.group_size else 0
-        for _ in range(d.n_layers):
+        for l in range(d.n_layers):
+            want = wanted(name) and (layers is None or l in layers)
             if d.group_size == 0:  # dense Linear (src/model.rs:11-15)
-                out.append(take(n_out * n_in, np.float32).reshape(n_out, n_in).astype(np.float64))
+                a = take(n_out * n_in, np.float32, want)
+                out.append(a.reshape(n_out, n_in).astype(np.float64) if want else None)
                 continue
-            qw = take(n_out * n_in // 8, np.int32).reshape(n_out, n_in // 8)
-            qz = take(n_out // 8 * g, np.int32).reshape(n_out // 8, g)
-            sc = take(n_out * g, np.float32).reshape(n_out, g)
-            gi = take(n_in, np.int32)
+            qw = take(n_out * n_in // 8, np.int32, want)
+            qz = take(n_out // 8 * g, np.int32, want)
+            sc = take(n_out * g, np.float32, want)
+            gi = take(n_in, np.int32, want)
+            if not want:
+                out.append(None)
+                continue
+            qw, qz, sc = qw.reshape(n_out, n_in // 8), qz.reshape(n_out // 8, g), sc.reshape(n_out, g)
+            idx = np.arange(n_out)
+            if max_rows and n_out > 2 * max_rows:
+                assert max_rows % 8 == 0
+                idx = np.concatenate([idx[:max_rows], idx[-max_rows:]])
+                qw, sc = qw[idx], sc[idx]
+                qz = np.concatenate([qz[:max_rows // 8], qz[-(max_rows // 8):]])
+            rows_of[name] = idx
             out.append(ck.dequant_bin(qw, qz, sc, gi, d.group_size))
         return out
 
+    def f64(name, n, shape):
+        a = take(n, np.float32, wanted(name))
+        return a.reshape(shape).astype(np.float64) if a is not None else None
+
     w = {"eps": float(take(1, np.float32)[0])}
-    w["emb"] = take(d.vocab_size * d.dim, np.float32).reshape(d.vocab_size, d.dim).astype(np.float64)
-    w["rms_att"] = take(d.n_layers * d.dim, np.float32).reshape(d.n_layers, d.dim).astype(np.float64)
-    w["wq"], w["wk"], w["wv"], w["wo"] = (qlin(d.dim, d.dim), qlin(d.dim, d.kv_dim),
-                                          qlin(d.dim, d.kv_dim), qlin(d.dim, d.dim))
-    w["rms_ffn"] = take(d.n_layers * d.dim, np.float32).reshape(d.n_layers, d.dim).astype(np.float64)
-    w["w1"], w["w2"], w["w3"] = (qlin(d.dim, d.hidden_dim), qlin(d.hidden_dim, d.dim),
-                                 qlin(d.dim, d.hidden_dim))
-    w["rms_final"] = take(d.dim, np.float32).astype(np.float64)
-    take(2 * d.seq_len * (d.head_size // 2), np.float32)
-    w["wcls"] = take(d.vocab_size * d.dim, np.float32).reshape(d.vocab_size, d.dim).astype(np.float64)
+    w["emb"] = f64("emb", d.vocab_size * d.dim, (d.vocab_size, d.dim))
+    w["rms_att"] = f64("rms_att", d.n_layers * d.dim, (d.n_layers, d.dim))
+    w["wq"], w["wk"], w["wv"], w["wo"] = (qlin("wq", d.dim, d.dim), qlin("wk", d.dim, d.kv_dim),
+                                          qlin("wv", d.dim, d.kv_dim), qlin("wo", d.dim, d.dim))
+    w["rms_ffn"] = f64("rms_ffn", d.n_layers * d.dim, (d.n_layers, d.dim))
+    w["w1"], w["w2"], w["w3"] = (qlin("w1", d.dim, d.hidden_dim), qlin("w2", d.hidden_dim, d.dim),
+                                 qlin("w3", d.dim, d.hidden_dim))
+    w["rms_final"] = f64("rms_final", d.dim, (d.dim,))
+    take(2 * d.seq_len * (d.head_size // 2), np.float32, False)
+    w["wcls"] = f64("wcls", d.vocab_size * d.dim, (d.vocab_size, d.dim))
     assert off[0] == img.nbytes
+    w["rows"] = rows_of
     return w
 
 
