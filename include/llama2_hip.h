@@ -164,6 +164,18 @@ void l2_qlinear_free(l2_qlinear *q);
  * x and y is not reproduced; the CPU path is the parity target). */
 int l2_qlinear_matvec(l2_qlinear *q, const float *x_host, int B, float *y_host);
 
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  x_dev f32[B][in] and
+ * y_dev f32[B][out] are DEVICE pointers; the gather and the matvec are enqueued on hip_stream (a
+ * hipStream_t; NULL is the default stream) and the call returns without waiting.  It calls no hipMalloc,
+ * hipFree or other allocating routine: the one intermediate (x in the layer's act-order) lives in a fixed
+ * device array of L2_MATVEC_DEVICE_MAX_ELEMS floats (4 MiB) that each GPU holds until the process
+ * ends, so B * in must not exceed that count (L2_ERR_RANGE otherwise).  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (two streams, two threads) race; serialise them.  y equals
+ * l2_qlinear_matvec's bit for bit. */
+#define L2_MATVEC_DEVICE_MAX_ELEMS (1u << 20)
+int l2_qlinear_matvec_device(l2_qlinear *q, const float *x_dev, int B, float *y_dev, void *hip_stream);
+
 /* The same operator on a projection of a loaded model: w.wq[layer].matvec(..). */
 int l2_model_qmatvec(l2_model *m, int layer, int proj, const float *x_host, int B, float *y_host);
 

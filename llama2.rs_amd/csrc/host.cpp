@@ -16,6 +16,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <mutex>
 #include <numeric>
 #include <thread>
 
@@ -954,6 +955,52 @@ extern "C" int l2_qlinear_matvec(l2_qlinear *q, const float *x_host, int B, floa
     if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
     L2_TRY(qlinear_scratch(q, B));
     return matvec_host(q->q, q->x, q->xg, q->y, x_host, B, y_host, q->stream);
+}
+
+// ---- the same operator for callers that cannot allocate ---------------------------------------------
+// (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The one buffer
+// l2_qlinear_matvec needs beyond its input and output -- x gathered into the layer's act-order -- lives in a
+// fixed device array instead of a hipMalloc'ed one.  Every GPU the library runs on holds its own copy of
+// the array, at its own address, until the process ends.
+static constexpr size_t kScratchFloats = L2_MATVEC_DEVICE_MAX_ELEMS; // 4 MiB
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+// The array's address on the current device.  `scratch` by name is a host-side stand-in, not a device
+// address; the address is asked for once per device, with that device current, and kept.
+static int scratch_ptr(float **out) {
+    static constexpr int kMaxDevices = 64;
+    static float *ptrs[kMaxDevices] = {};
+    static std::mutex mu;
+    int dev = 0;
+    L2_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return l2_fail(L2_ERR_HIP, "device %d: more devices than the scratch table holds", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return l2_fail(L2_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        ptrs[dev] = (float *)p;
+    }
+    *out = ptrs[dev];
+    return L2_OK;
+}
+
+extern "C" int l2_qlinear_matvec_device(l2_qlinear *q, const float *x_dev, int B, float *y_dev, void *hip_stream) {
+    if (!q || !x_dev || !y_dev) return l2_fail(L2_ERR_ARG, "null argument");
+    if (B < 1 || B > 4096) return l2_fail(L2_ERR_RANGE, "batch %d (1..4096)", B);
+    if ((size_t)B * (size_t)q->q.in > kScratchFloats)
+        return l2_fail(L2_ERR_RANGE, "B * in = %zu floats exceed the fixed scratch of %zu (no allocation is made here: "
+                                     "use a smaller batch, or l2_qlinear_matvec)",
+                       (size_t)B * (size_t)q->q.in, kScratchFloats);
+    float *xg = nullptr;
+    L2_TRY(scratch_ptr(&xg));
+    hipStream_t st = (hipStream_t)hip_stream;
+    // Every element of xg[0 .. B * in) is written by the gather before the matvec reads it: nothing of the
+    // previous call's contents is read, so nothing needs clearing.
+    L2_TRY(gather_launch(xg, x_dev, q->q.g_index, q->q.in, B, st));
+    L2_TRY(q4_one(q->q, xg, y_dev, B, st));
+    return L2_OK;
 }
 
 static int op_scratch(l2_model *m, size_t elems) {

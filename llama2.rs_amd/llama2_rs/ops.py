@@ -86,6 +86,13 @@ class QLinear:
         check(lib().l2_qlinear_matvec(self.h, _p(xb), xb.shape[0], _p(y)))
         return y[0] if one else y
 
+    def matvec_device(self, x_dev: int, B: int, y_dev: int, stream: int = 0) -> None:
+        """The same operator on DEVICE pointers (addresses as integers), enqueued on `stream` (a hipStream_t
+        as an integer, 0 = the default stream) without waiting and without allocating anything: for callers
+        under graph capture or in a serving loop.  B * in is bounded by the library's fixed scratch."""
+        check(lib().l2_qlinear_matvec_device(self.h, C.c_void_p(x_dev), B, C.c_void_p(y_dev),
+                                             C.c_void_p(stream) if stream else None))
+
     def close(self):
         if self.h:
             lib().l2_qlinear_free(self.h)
