@@ -11,6 +11,14 @@ prompt positions (forced tokens through the same B=1 loop); the K timed steps
 are greedy decode steps with the argmax fed back on the device.  Weights and
 KV cache are resident in HBM before the timed region starts.
 
+The top level of the JSON line is that run (K and W as given).  Beside it, in
+the same process and the same line, "configs" carries the stated workloads at
+their stated lengths: the 7B decode of 256 tokens after a 16-token prompt, the
+7B prefill of a 512-token prompt in chunks of 128 through the MFMA path, the
+13B decode (32 + 256), and the 70B group-64 decode of 128 tokens behind 4096
+cached positions, each with its own roofline object (--configs none skips
+them, --configs 1,4 selects).
+
 Prints ONE JSON line.
 """
 from __future__ import annotations
@@ -18,6 +26,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,13 +35,8 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "llama2.rs_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
-
-# HBM bytes per layer moved by the four q4 launches, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (each scaled by the reading of the plain copy kernel of known size in the same run):
-# the summaries are profiles/q4_matvec_<model>_decode_hbm_counters.txt.
-MEASURED_Q4_TRAFFIC_PER_LAYER = {
-    "7B": 49226169 + 2 * 18683076 + 24774068 + 234963 + 2 * 125403 + 265887,
-}
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix peak
+Q4_CLASSES = ["q4_qkv", "q4_wo", "q4_w13", "q4_w2"]
 
 
 def q4_bytes(n_in: int, n_out: int, G: int) -> int:
@@ -63,15 +67,167 @@ def token_bytes(d, pos: int) -> int:
     return d.n_layers * per_layer + cb["classifier"] + d.dim * 4 + d.dim * 4 + kv
 
 
-MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix peak
+def measured_traffic(model: str, kernels: dict):
+    """Mean HBM bytes per q4 launch of a layer from the committed rocprofv3 counter summary
+    profiles/q4_matvec_<model>_decode_hbm_counters.txt (FETCH_SIZE + WRITE_SIZE per dispatch, already scaled
+    to bytes there), matched by kernel name against the kernels this build launches.  Returns
+    (bytes or None, note): None with the reason when the summary is missing or names another build's kernels."""
+    path = os.path.join(ROOT, "profiles", f"q4_matvec_{model}_decode_hbm_counters.txt")
+    if not os.path.exists(path):
+        return None, f"no counter summary profiles/{os.path.basename(path)}"
+    table = {"FETCH_SIZE": {}, "WRITE_SIZE": {}}
+    section = None
+    for line in open(path):
+        m = re.match(r"^(FETCH_SIZE|WRITE_SIZE):", line)
+        if m:
+            section = m.group(1)
+            continue
+        m = re.match(r"^\s+(\d+)\s+([\d.]+)\s+(\d+)\s+(\S.*)$", line)
+        if m and section:
+            table[section][m.group(4).strip()] = int(m.group(3))
+    total = 0
+    for cls in Q4_CLASSES:
+        name = kernels.get(cls, "?") + "(Q4Launch)"
+        for section in ("FETCH_SIZE", "WRITE_SIZE"):
+            if name not in table[section]:
+                return None, (f"profiles/{os.path.basename(path)} holds no {section} reading for {name} ({cls}): "
+                              "it was taken with other kernels, take it again")
+            total += table[section][name]
+    return round(total / len(Q4_CLASSES)), f"profiles/{os.path.basename(path)}"
 
 
-def prefill_workload(a, d, m, img, np) -> int:
-    """BASELINE config 2: a prompt of --prompt-len random ids prefilled in chunks of --chunk tokens
-    through the dequant->fp16 MFMA GEMM path, followed by --steps greedy decode steps."""
+class Loaded:
+    """A random-init model of one preset resident on the GPU, with its host image (the CPU baseline reads it)."""
+
+    def __init__(self, ops, name: str, group: int, layers: int, max_seq: int, seed: int):
+        from llama2_rs import checkpoint as ck
+        self.ops, self.name, self.seed = ops, name, seed
+        d = ops.preset(name, group or (64 if name == "70B" else 128))
+        if layers:
+            d = ck.Dims(d.dim, d.hidden_dim, layers, d.n_heads, d.n_kv_heads, d.vocab_size, d.seq_len, d.group_size)
+        self.d = d
+        self.max_seq = max(d.seq_len, max_seq)
+        t0 = time.time()
+        self.img = ops.synth_image(d, seed)
+        self.t_synth = time.time() - t0
+        t0 = time.time()
+        self.m = ops.Model(self.img, d, max_seq=self.max_seq)
+        self.t_upload = time.time() - t0
+        self.label = f"Llama-2-{name} GPTQ 4-bit group {d.group_size} act-order, random-init" + \
+                     (f", {layers} of its layers" if layers else "")
+
+    def close(self):
+        self.m.close()
+        self.img = None
+
+
+def decode_run(np, M: Loaded, W: int, K: int, pos0: int, cpu: bool, cpu_tokens: int) -> dict:
+    """W prompt positions forced through the B=1 loop (untimed), then K greedy steps timed; the q4 roofline from
+    per-dispatch events of further steps; optionally the CPU restatement on a bounded sample of the same run."""
+    m, d = M.m, M.d
+    rng = np.random.default_rng(M.seed)
+    prompt = rng.integers(0, d.vocab_size, size=W).astype(np.int32)
+    m.reset()
+    if pos0:
+        m.fill_kv_synthetic(0, pos0, seed=M.seed)
+    tok = 1
+    for i in range(W):
+        m.decode_greedy(tok, pos0 + i)
+        tok = int(prompt[i])
+    t0 = time.perf_counter()
+    ids, ms_events = m.decode_bench(tok, pos0 + W, K)
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    tok_s = K / (wall_ms * 1e-3)
+
+    n_prof = min(8, K)
+    prof = m.decode_profile(int(ids[-1]), pos0 + W + K, n_prof) if pos0 + W + K + n_prof <= M.max_seq else {}
+    cb = class_bytes(d)
+    kern = {}
+    for c in Q4_CLASSES + ["classifier", "attention"]:
+        if c in prof and prof[c][1] > 0:
+            us = prof[c][0] / prof[c][1] * 1e3
+            kern[c] = {"us": round(us, 2)}
+            if c in cb:
+                kern[c].update({"bytes": cb[c], "GBs": round(cb[c] / us / 1e3, 1)})
+    roofline = None
+    if all(c in kern for c in Q4_CLASSES):
+        tot_b = sum(cb[c] * prof[c][1] for c in Q4_CLASSES)
+        tot_ms = sum(prof[c][0] for c in Q4_CLASSES)
+        achieved = tot_b / (tot_ms * 1e-3) / 1e9
+        traffic, note = measured_traffic(M.name, m.q4_kernels())
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    # mean HBM bytes per q4 launch (a layer has four), beside the algorithmic mean
+                    "traffic": traffic, "traffic_source": note,
+                    "algorithmic_bytes_per_launch": round(sum(cb[c] for c in Q4_CLASSES) / 4),
+                    "kernel": "q4 matvec: the four q4 launches of a layer (q|k|v, wo, w1|w3, w2), durations from "
+                              "the dispatches' own start/stop events",
+                    "per_launch": kern}
+    mid = pos0 + W + K // 2
+    out = {
+        "workload": (f"{M.label}; batch-1 greedy decode of {K} tokens after a {W}-token random prompt"
+                     + (f", KV cache pre-filled to {pos0} positions" if pos0 else "")),
+        "value": round(tok_s, 2), "unit": "tok/s", "steps": K, "warmup": W,
+        "ms_per_step": round(wall_ms / K, 4), "event_ms_per_step": round(ms_events / K, 4),
+        "bytes_per_token": token_bytes(d, mid),
+        "decode_GBs": round(token_bytes(d, mid) * tok_s / 1e9, 1),
+        "decode_frac_of_hbm_peak": round(token_bytes(d, mid) * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+        "roofline": roofline,
+    }
+    if cpu:
+        from oracle import oracle_lib
+        o = oracle_lib.Model(M.img, d, max_seq=M.max_seq)
+        cores = oracle_lib.num_threads()
+        o.new_state()
+        if pos0:
+            kc, vc = o.kv_cache()
+            for l in range(d.n_layers):
+                k, v = m.read_kv(l, 0, pos0)
+                kc[l, :pos0] = k
+                vc[l, :pos0] = v
+        # bounded sample of the same workload: the prompt (at most 4 positions of it timed here, the rest
+        # taken from the GPU's cache, which the parity tests hold equal), then n_cpu greedy tokens
+        w_cpu = min(W, 4)
+        if W > w_cpu:
+            kc, vc = o.kv_cache()
+            for l in range(d.n_layers):
+                k, v = m.read_kv(l, pos0, W - w_cpu)
+                kc[l, pos0:pos0 + W - w_cpu] = k
+                vc[l, pos0:pos0 + W - w_cpu] = v
+        tokc = 1 if W == w_cpu else int(prompt[W - w_cpu - 1])
+        t0 = time.perf_counter()
+        for i in range(W - w_cpu, W):
+            o.transformer([tokc], [pos0 + i])
+            tokc = int(prompt[i])
+        t_prompt = time.perf_counter() - t0
+        n_cpu = cpu_tokens
+        if n_cpu <= 0:
+            per_tok = max(t_prompt / w_cpu, 1e-3) if w_cpu else 1.0
+            n_cpu = int(max(4, min(K, 15.0 / per_tok)))
+        cpu_ids = []
+        t0 = time.perf_counter()
+        for i in range(n_cpu):
+            logits = o.transformer([tokc], [pos0 + W + i])
+            tokc = oracle_lib.argmax(logits)
+            cpu_ids.append(tokc)
+        t_dec = time.perf_counter() - t0
+        same = int(np.sum(np.cumprod(np.asarray(cpu_ids) == ids[:n_cpu])))
+        out["cpu_baseline"] = {
+            "value": round(n_cpu / t_dec, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "sample": (f"C restatement of the reference CPU path (OpenMP over rows/heads, 8-lane AVX2), same weights, "
+                       f"prompt and cache: {n_cpu} greedy tokens of the {K}; decode-only timing"),
+        }
+        out["greedy_tokens_identical_to_cpu"] = f"{same}/{n_cpu}"
+        o.close()
+    return out
+
+
+def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool) -> dict:
+    """BASELINE config 2: a prompt of n random ids prefilled in chunks through the dequant->fp16 MFMA GEMM path,
+    followed by K greedy decode steps."""
     from llama2_rs import _lib
-    n, chunk, K = a.prompt_len, a.chunk, a.steps
-    rng = np.random.default_rng(a.seed)
+    m, d = M.m, M.d
+    rng = np.random.default_rng(M.seed)
     prompt = rng.integers(0, d.vocab_size, size=n).astype(np.int32)
     flops_per_token = 2 * d.n_layers * (2 * d.dim * d.dim + 2 * d.dim * d.kv_dim + 3 * d.dim * d.hidden_dim)
 
@@ -89,29 +245,27 @@ def prefill_workload(a, d, m, img, np) -> int:
 
     t_mfma = run(_lib.PREFILL_MFMA)
     ids, ms_dec = m.decode_bench(int(prompt[-1]), n, K)
-    t_fp32 = run(_lib.PREFILL_FP32) if a.cpu_tokens >= 0 else None
-    ids32, _ = m.decode_bench(int(prompt[-1]), n, K)
-    same = int(np.sum(np.cumprod(ids == ids32)))
+    out = {}
+    if compare_fp32:
+        t_fp32 = run(_lib.PREFILL_FP32)
+        ids32, _ = m.decode_bench(int(prompt[-1]), n, K)
+        out["fp32_path_tok_s"] = round(n / t_fp32, 1)
+        out["greedy_tokens_same_as_after_fp32_prefill"] = f"{int(np.sum(np.cumprod(ids == ids32)))}/{K}"
+    m.set_prefill_mode(_lib.PREFILL_FP32)
     tok_s = n / t_mfma
     tflops = flops_per_token * tok_s / 1e12
-    result = {
-        "metric": f"{a.model} q4 prefill tok/s on 1 MI355X", "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1,
-        "steps": n // chunk, "warmup": 1, "ms_per_step": round(t_mfma * 1e3 / max(1, (n + chunk - 1) // chunk), 3),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 x f16 -> f32 (MFMA)",
-        "data": "synthetic",
-        "config": {"workload": f"Llama-2-{a.model} GPTQ 4-bit group {d.group_size} act-order, random-init; {n}-token random "
-                               f"prompt prefilled in chunks of {chunk} through the dequant->fp16 MFMA GEMM, then {K} greedy steps",
-                   "seed": a.seed},
+    n_chunks = (n + chunk - 1) // chunk
+    out.update({
+        "workload": f"{M.label}; {n}-token random prompt prefilled in chunks of {chunk} through the dequant->fp16 "
+                    f"MFMA GEMM, then {K} greedy steps",
+        "value": round(tok_s, 1), "unit": "tok/s", "steps": n_chunks, "warmup": 1,
+        "ms_per_step": round(t_mfma * 1e3 / n_chunks, 3), "dtype": "f16 x f16 -> f32 (MFMA)",
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
                      "flops_per_token": flops_per_token},
-        "fp32_path_tok_s": round(n / t_fp32, 1) if t_fp32 else None,
         "decode_after_prefill_tok_s": round(K / (ms_dec * 1e-3), 1),
-        "greedy_tokens_same_as_after_fp32_prefill": f"{same}/{K}",
-    }
-    m.close()
-    print(json.dumps(result))
-    return 0
+    })
+    return out
 
 
 def main() -> int:
@@ -122,15 +276,21 @@ def main() -> int:
                     help="untimed steps = the prompt, forced through the loop (default 16; 32 for 13B, as its config asks)")
     ap.add_argument("--model", default="7B", choices=["7B", "13B", "70B"])
     ap.add_argument("--group", type=int, default=0, help="group size (default: 128, 64 for 70B)")
+    ap.add_argument("--layers", type=int, default=0,
+                    help="keep only this many layers of the architecture (same kernels and shapes per launch; for "
+                         "counter runs and quick checks, never a headline)")
     ap.add_argument("--kv-prefill", type=int, default=0,
                     help="fill this many cache positions synthetically before the prompt (70B long-context case)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-tokens", type=int, default=0, help="decoded tokens of the CPU sample (0 = sized to ~20 s)")
+    ap.add_argument("--cpu-tokens", type=int, default=0, help="decoded tokens of the CPU sample (0 = sized to ~15 s)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
-                    help="prefill: BASELINE config 2 (prompt in chunks through the dequant->fp16 MFMA GEMM, then decode)")
+                    help="prefill: BASELINE config 2 alone (prompt in chunks through the dequant->fp16 MFMA GEMM, then decode)")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--chunk", type=int, default=128)
+    ap.add_argument("--configs", default=None,
+                    help="which of the stated workloads to run beside the headline: comma list of 1,2,3,4, or none "
+                         "(default: all for the plain 7B run, none otherwise)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no sharding, no collectives); "
@@ -142,28 +302,26 @@ def main() -> int:
     if K < 1 or W < 0:
         print("bench.py: --steps must be >= 1 and --warmup >= 0", file=sys.stderr)
         return 2
+    plain = a.model == "7B" and not a.layers and not a.group and not a.kv_prefill and a.workload == "decode"
+    if a.configs is None:
+        a.configs = "1,2,3,4" if plain else "none"
+    want = set() if a.configs == "none" else {int(c) for c in a.configs.split(",") if c}
 
     import numpy as np
     from llama2_rs import ops
 
-    G = a.group or (64 if a.model == "70B" else 128)
-    d = ops.preset(a.model, G)
-    max_seq = max(d.seq_len, a.kv_prefill + W + K + 8)
-    t0 = time.time()
-    img = ops.synth_image(d, a.seed)
-    t_synth = time.time() - t0
-    t0 = time.time()
-    m = ops.Model(img, d, max_seq=max_seq)
-    t_upload = time.time() - t0
+    M = Loaded(ops, a.model, a.group, a.layers, a.kv_prefill + max(W + K, 16 + 256) + 16, a.seed)
 
     if a.workload == "prefill":
-        return prefill_workload(a, d, m, img, np)
-
-    rng = np.random.default_rng(a.seed)
-    prompt = rng.integers(0, d.vocab_size, size=W).astype(np.int32)
-    pos0 = a.kv_prefill
-    if pos0:
-        m.fill_kv_synthetic(0, pos0, seed=a.seed)
+        r = prefill_run(np, M, a.prompt_len, a.chunk, K, not a.no_cpu_baseline)
+        result = {"metric": f"{a.model} q4 prefill tok/s on 1 MI355X", "value": r["value"], "unit": "tok/s", "n_gpus": 1,
+                  "steps": r["steps"], "warmup": 1, "ms_per_step": r["ms_per_step"], "higher_is_better": True,
+                  "scaling": "weak", "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic",
+                  "config": {"workload": r["workload"], "seed": a.seed}}
+        result.update({k: v for k, v in r.items() if k not in result and k != "workload"})
+        M.close()
+        print(json.dumps(result))
+        return 0
 
     # plain device copy of known size: the box's copy bandwidth, and the known-size
     # kernel that counter readings are scaled by
@@ -171,109 +329,38 @@ def main() -> int:
     copy_ms = ops.copy_bench(copy_bytes, 8)
     copy_gbs = 2 * copy_bytes * 8 / (copy_ms * 1e-3) / 1e9
 
-    # warm-up: the prompt positions, forced through the B=1 loop
-    tok = 1
-    for i in range(W):
-        m.decode_greedy(tok, pos0 + i)
-        tok = int(prompt[i])
-    # timed: K greedy steps, argmax fed back on the device
-    t0 = time.perf_counter()
-    ids, ms_events = m.decode_bench(tok, pos0 + W, K)
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    tok_s = K / (wall_ms * 1e-3)
-
-    # per-launch event timing of the same loop, for the roofline of the dominant kernel
-    n_prof = min(8, K)
-    prof = m.decode_profile(int(ids[-1]), pos0 + W + K, n_prof) if pos0 + W + K + n_prof <= max_seq else {}
-    cb = class_bytes(d)
-    q4_classes = ["q4_qkv", "q4_wo", "q4_w13", "q4_w2"]
-    kern = {}
-    for c in q4_classes + ["classifier"]:
-        if c in prof and prof[c][1] > 0:
-            us = prof[c][0] / prof[c][1] * 1e3
-            kern[c] = {"us": round(us, 2), "bytes": cb[c], "GBs": round(cb[c] / us / 1e3, 1)}
-    roofline = None
-    if all(c in kern for c in q4_classes):
-        tot_b = sum(cb[c] * prof[c][1] for c in q4_classes)
-        tot_ms = sum(prof[c][0] for c in q4_classes)
-        achieved = tot_b / (tot_ms * 1e-3) / 1e9
-        traffic = MEASURED_Q4_TRAFFIC_PER_LAYER.get(a.model)
-        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4),
-                    # mean HBM bytes per q4 launch (a layer has four), beside the algorithmic mean
-                    "traffic": round(traffic / 4) if traffic else None,
-                    "algorithmic_bytes_per_launch": round(sum(cb[c] for c in q4_classes) / 4),
-                    "kernel": "q4 matvec: the four q4 launches of a layer (q|k|v, wo, w1|w3, w2), durations from "
-                              "the dispatches' own start/stop events",
-                    "per_launch": kern}
-
+    r = decode_run(np, M, W, K, a.kv_prefill, not a.no_cpu_baseline, a.cpu_tokens)
     result = {
         "metric": f"{a.model} q4 decode tok/s on 1 MI355X",
-        "value": round(tok_s, 2),
-        "unit": "tok/s",
-        "n_gpus": 1,
-        "steps": K,
-        "warmup": W,
-        "ms_per_step": round(wall_ms / K, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {
-            "workload": (f"Llama-2-{a.model} GPTQ 4-bit group {G} act-order, random-init; batch-1 greedy decode of "
-                         f"{K} tokens after a {W}-token random prompt"
-                         + (f", KV cache pre-filled to {pos0} positions" if pos0 else "")),
-            "seed": a.seed, "max_seq": max_seq,
-        },
-        "event_ms_per_step": round(ms_events / K, 4),
-        "bytes_per_token": token_bytes(d, pos0 + W + K // 2),
-        "decode_GBs": round(token_bytes(d, pos0 + W + K // 2) * tok_s / 1e9, 1),
-        "decode_frac_of_hbm_peak": round(token_bytes(d, pos0 + W + K // 2) * tok_s / 1e9 / HBM_PEAK_GBS, 4),
-        "roofline": roofline,
-        "copy_GBs": round(copy_gbs, 1),
-        "setup_s": {"synth": round(t_synth, 1), "upload": round(t_upload, 1)},
+        "value": r["value"], "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": r["workload"], "seed": a.seed, "max_seq": M.max_seq},
     }
+    result.update({k: v for k, v in r.items() if k not in result and k != "workload"})
+    result["copy_GBs"] = round(copy_gbs, 1)
+    result["setup_s"] = {"synth": round(M.t_synth, 1), "upload": round(M.t_upload, 1)}
 
-    if not a.no_cpu_baseline:
-        from oracle import oracle_lib
-        o = oracle_lib.Model(img, d, max_seq=max_seq)
-        cores = oracle_lib.num_threads()
-        # bounded sample of the same workload: the same prompt, then n_cpu greedy tokens
-        n_cpu = a.cpu_tokens
-        o.new_state()
-        if pos0:
-            kc, vc = o.kv_cache()
-            for l in range(d.n_layers):
-                k, v = m.read_kv(l, 0, pos0)
-                kc[l, :pos0] = k
-                vc[l, :pos0] = v
-        tokc = 1
-        t0 = time.perf_counter()
-        for i in range(W):
-            o.transformer([tokc], [pos0 + i])
-            tokc = int(prompt[i])
-        t_prompt = time.perf_counter() - t0
-        if n_cpu <= 0:
-            per_tok = max(t_prompt / max(W, 1), 1e-3) if W else 1.0
-            n_cpu = int(max(4, min(K, 20.0 / per_tok - W)))
-        cpu_ids = []
-        t0 = time.perf_counter()
-        for i in range(n_cpu):
-            logits = o.transformer([tokc], [pos0 + W + i])
-            tokc = oracle_lib.argmax(logits)
-            cpu_ids.append(tokc)
-        t_dec = time.perf_counter() - t0
-        same = int(np.sum(np.cumprod(np.asarray(cpu_ids) == ids[:n_cpu])))
-        result["cpu_baseline"] = {
-            "value": round(n_cpu / t_dec, 3), "unit": "tok/s", "cores": cores, "kind": "port",
-            "sample": (f"C restatement of the reference CPU path (OpenMP over rows/heads, 8-lane AVX2), same weights and "
-                       f"prompt: {W} prompt positions then {n_cpu} greedy tokens of the {K}; decode-only timing"),
-        }
-        result["greedy_tokens_identical_to_cpu"] = f"{same}/{n_cpu}"
-        o.close()
-
-    m.close()
+    configs = {}
+    if want:
+        t_all = time.time()
+        if 1 in want:   # config 1 at its stated length
+            configs["cfg1_7B_decode_16+256"] = decode_run(np, M, 16, 256, 0, False, 0)
+        if 2 in want:   # config 2: 512-token prompt in chunks of 128 through the MFMA path, then 64 greedy steps
+            configs["cfg2_7B_prefill_512_by_128"] = prefill_run(np, M, 512, 128, 64, False)
+        M.close()
+        if 3 in want:
+            M3 = Loaded(ops, "13B", 0, 0, 32 + 256 + 16, a.seed)
+            configs["cfg3_13B_decode_32+256"] = decode_run(np, M3, 32, 256, 0, False, 0)
+            M3.close()
+        if 4 in want:   # the configuration the 60 % target is stated on
+            M4 = Loaded(ops, "70B", 0, 0, 4096 + 4 + 128 + 16, a.seed)
+            configs["cfg4_70B_g64_decode_128_behind_4096"] = decode_run(np, M4, 4, 128, 4096, not a.no_cpu_baseline, 8)
+            M4.close()
+        result["configs"] = configs
+        result["configs_wall_s"] = round(time.time() - t_all, 1)
+    else:
+        M.close()
     print(json.dumps(result))
     return 0
 

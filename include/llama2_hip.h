@@ -263,6 +263,12 @@ const char *l2_kernel_class_name(int cls);
 int l2_decode_profile(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
                       float *ms_by_class, int32_t *launches_by_class);
 
+/* Which kernel each q4 launch class of the decode step runs for this model, as
+ * "q4_qkv=<kernel>;q4_wo=<kernel>;q4_w13=<kernel>;q4_w2=<kernel>;" with the names a profiler prints
+ * (template arguments included), so that counter readings taken per kernel name can be matched to the
+ * launches of a run.  Launches nothing. */
+int l2_model_q4_kernels(l2_model *m, char *out, size_t cap);
+
 /* Plain device-to-device copy of nbytes, iters times: the box's achievable
  * copy bandwidth (bytes moved = 2*nbytes per iteration). */
 int l2_copy_bench(size_t nbytes, int iters, float *ms_total);

@@ -27,6 +27,7 @@
 
 static thread_local char g_err[512] = "";
 thread_local Q4ProfHook g_q4_prof;
+thread_local Q4NameHook g_q4_name;
 
 int l2_fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -330,10 +331,6 @@ static constexpr int kMaxSplits = 64;
 // failed, or that nobody recorded, are destroyed here and leave no record.
 template <class F>
 static int timed_launch(l2_model *m, int cls, F &&launch) {
-    static const bool tile_form = []() {
-        const char *v = getenv("L2_Q4_IMPL");
-        return v && !strcmp(v, "tile");
-    }();
     l2_model::ProfRec r{cls, nullptr, nullptr};
     auto drop = [&]() {
         if (r.e0) (void)hipEventDestroy(r.e0);
@@ -345,7 +342,7 @@ static int timed_launch(l2_model *m, int cls, F &&launch) {
         drop();
         return l2_fail(L2_ERR_HIP, "hipEventCreate: %s", hipGetErrorString(e));
     }
-    const bool q4 = !tile_form && m->d.group_size != 0 &&
+    const bool q4 = m->d.group_size != 0 &&
                     (cls == K_Q4_QKV || cls == K_Q4_WO || cls == K_Q4_W13 || cls == K_Q4_W2);
     int rc = L2_OK;
     bool recorded = true;
@@ -1645,6 +1642,54 @@ extern "C" int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t 
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (out_ids) L2_HIP(hipMemcpy(out_ids, m->dout_ids, (size_t)n_tokens * 4, hipMemcpyDeviceToHost));
+    return L2_OK;
+}
+
+// Which kernel each q4 launch class of this model's decode step runs: "class=kernel;..." with the kernel's
+// name as a profiler prints it (template arguments included).  Nothing is launched.
+extern "C" int l2_model_q4_kernels(l2_model *m, char *out, size_t cap) {
+    if (!m || !out || cap < 2) return l2_fail(L2_ERR_ARG, "bad argument");
+    out[0] = '\0';
+    if (m->d.group_size == 0) return L2_OK; // the model without quantisation has no q4 launches
+    const int layer = 0;
+    const DevQLinear &wq = m->q[L2_WQ][layer], &wk = m->q[L2_WK][layer], &wv = m->q[L2_WV][layer],
+                     &wo = m->q[L2_WO][layer], &w1 = m->q[L2_W1][layer], &w2 = m->q[L2_W2][layer],
+                     &w3 = m->q[L2_W3][layer];
+    const float *some = (const float *)m->dimage; // only null / non-null matters for the choice of kernel
+    struct { const char *cls; Q4Launch L; } items[4];
+    items[0].cls = "q4_qkv";
+    items[0].L = launch_of(wq, 1, m->rms_eps);
+    items[0].L.m[0] = mat_of(wq, some, some, nullptr);
+    items[0].L.m[1] = mat_of(wk, some, some, nullptr);
+    items[0].L.m[2] = mat_of(wv, some, some, nullptr);
+    items[0].L.n_mats = 3;
+    items[1].cls = "q4_wo";
+    items[1].L = launch_of(wo, 1, 0.f);
+    items[1].L.m[0] = mat_of(wo, some, nullptr, nullptr);
+    items[2].cls = "q4_w13";
+    items[2].L = launch_of(w1, 1, m->rms_eps);
+    items[2].L.m[0] = mat_of(w1, some, some, nullptr);
+    items[2].L.m[1] = mat_of(w3, some, some, nullptr);
+    items[2].L.n_mats = 2;
+    items[2].L.pair = 1;
+    items[3].cls = "q4_w2";
+    items[3].L = launch_of(w2, 1, 0.f);
+    items[3].L.m[0] = mat_of(w2, some, nullptr, nullptr);
+    std::string all;
+    for (auto &it : items) {
+        char name[160] = "";
+        g_q4_name.buf = name;
+        g_q4_name.cap = (int)sizeof(name);
+        g_q4_name.armed = true;
+        const int rc = q4_matvec_launch(it.L, m->stream);
+        const bool answered = !g_q4_name.armed;
+        g_q4_name.armed = false;
+        L2_TRY(rc);
+        if (!answered) return l2_fail(L2_ERR_ARG, "the launcher of %s did not name its kernel", it.cls);
+        all += std::string(it.cls) + "=" + name + ";";
+    }
+    if (all.size() + 1 > cap) return l2_fail(L2_ERR_ARG, "buffer of %zu bytes, %zu needed", cap, all.size() + 1);
+    memcpy(out, all.c_str(), all.size() + 1);
     return L2_OK;
 }
 

@@ -33,6 +33,8 @@
 // (src/models.rs:271-276) delivered in w2's input order.
 #include <string.h>
 
+#include <stdio.h>
+
 #include "q4_common.h"
 
 namespace {
@@ -219,6 +221,11 @@ int launch_t(Q4Launch &L, hipStream_t stream) {
     const int C = L.in / 32;
     const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
     auto kern = q4_matvec_kernel<G, R, NW, PAIR>;
+    if (g_q4_name.armed) {
+        g_q4_name.armed = false;
+        snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_matvec_kernel<%d, %d, %d, %s>", G, R, NW, PAIR ? "true" : "false");
+        return L2_OK;
+    }
     if (lds + 256 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
     if (lds > 64 * 1024) {
         static size_t raised = 0; // per instantiation: the largest dynamic LDS size allowed so far

@@ -25,6 +25,7 @@
 //   sum_k (n_k - z1) x_k = delta * (I - (z1 - 8) * sum_k q_k),  I = sum_d 16^d a_d.
 // The quantisation error (2^-23 of the chunk maximum per element) is of the size of fp32 rounding.  Its
 // quantisation prologue costs more than the shorter loop saves on the shapes measured, hence not the default.
+#include <stdio.h>
 #include <string.h>
 
 #include "q4_common.h"
@@ -516,6 +517,12 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     L.rows_per_block = rpb;
     for (int i = 0; i < L.n_mats; i++) L.m[i].row_blocks = (L.m[i].out + rpb - 1) / rpb;
     auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE, P>;
+    if (g_q4_name.armed) {
+        g_q4_name.armed = false;
+        snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_stream_kernel<%d, %d, %d, %s, %d, %d>", G, NWK, S,
+                 PAIR ? "true" : "false", MODE, P);
+        return L2_OK;
+    }
     if (lds > 48 * 1024) {
         static size_t raised = 0; // per instantiation
         if (lds > raised) {

@@ -109,6 +109,15 @@ struct Q4ProfHook {
 };
 extern thread_local Q4ProfHook g_q4_prof;
 
+// When armed, the next q4 launch is not launched: the launcher writes the name of the kernel it would run
+// (as a profiler prints it, template arguments included) into buf and disarms the hook.
+struct Q4NameHook {
+    char *buf = nullptr;
+    int cap = 0;
+    bool armed = false;
+};
+extern thread_local Q4NameHook g_q4_name;
+
 // Launch the fp32 dequant matvec for up to 3 matrices that share `in`
 // (wq|wk|wv), or a (w1, w3) pair.  Fills row_blocks itself.
 int q4_matvec_launch(Q4Launch &L, hipStream_t stream);

@@ -67,6 +67,7 @@ SIGNATURES = {
     "l2_qlinear_free": (None, [_VP]),
     "l2_qlinear_matvec": (_I, [_VP, _VP, _I, _VP]),
     "l2_qlinear_matvec_device": (_I, [_VP, _VP, _I, _VP, _VP]),
+    "l2_model_q4_kernels": (_I, [_VP, C.c_char_p, _SZ]),
     "l2_model_qmatvec": (_I, [_VP, _I, _I, _VP, _I, _VP]),
     "l2_model_classifier": (_I, [_VP, _VP, _VP]),
     "l2_forward": (_I, [_VP, _VP, _VP, _VP, _I, _VP]),

@@ -213,6 +213,12 @@ class Model:
         check(lib().l2_decode_profile(self.h, self.state, token, pos, n_tokens, _p(ms), _p(cnt)))
         return {lib().l2_kernel_class_name(i).decode(): (float(ms[i]), int(cnt[i])) for i in range(n)}
 
+    def q4_kernels(self) -> dict:
+        """{launch class: kernel name as a profiler prints it} of this model's decode step."""
+        buf = C.create_string_buffer(1024)
+        check(lib().l2_model_q4_kernels(self.h, buf, 1024))
+        return dict(item.split("=", 1) for item in buf.value.decode().split(";") if item)
+
     def read_kv(self, layer: int, pos0: int, npos: int):
         d = self.dims
         k = np.empty((npos, d.n_kv_heads, d.head_size), np.float32)
