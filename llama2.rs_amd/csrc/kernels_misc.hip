@@ -150,6 +150,8 @@ __device__ __forceinline__ unsigned long long amax_key(float v, int idx) {
 // the end re-read the row's last 16 bytes against a zero of x, rows past the
 // end re-read the last row.  Inputs longer than 32 * 64 float4 take several
 // such passes over a row (R = 1) into the same accumulator.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 template <int KI> // float4 per lane, row and pass
 __global__ __launch_bounds__(256) void dense_matvec_kernel(const DenseArgs A) {
     constexpr int R = 32 / KI >= 1 ? 32 / KI : 1;
@@ -207,7 +209,9 @@ __global__ __launch_bounds__(256) void dense_matvec_kernel(const DenseArgs A) {
 #pragma unroll
             for (int i = 0; i < KI; i++) {
                 const uint32_t col = (uint32_t)min((pass * KI + i) * 64 + lane, n4 - 1) << 4;
-                wv[k][i] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(w4) + (row + col));
+                // read once per token: non-temporal, so that the rows do not displace what is re-read
+                wv[k][i] = __builtin_bit_cast(float4, __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(
+                                                          reinterpret_cast<const char *>(w4) + (row + col))));
             }
         }
     };

@@ -26,6 +26,7 @@
 // The quantisation error (2^-23 of the chunk maximum per element) is of the size of fp32 rounding.  Its
 // quantisation prologue costs more than the shorter loop saves on the shapes measured, hence not the default.
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "q4_common.h"
@@ -121,13 +122,54 @@ __device__ __forceinline__ float chunk_idot(const uint4 w, const int (&xp)[24]) 
     return fmaf((float)hi, 4096.0f, (float)lo);
 }
 
+// A load of weights: read once per token and never again before some 40 GB of other weights have gone by,
+// so it is marked non-temporal (no point in keeping the line in L2 or in the memory-side cache, where it
+// would only push out what is re-read: x, the scales' neighbours, the next kernel's operands).  Measured on
+// the 70B shapes: w1|w3 51.0 -> 45.8 us, w2 28.7 -> 25.7 us per launch.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 template <class T>
 __device__ __forceinline__ T ld_at(const void *base, uint32_t byte_offset) {
-    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_offset);
+    const char *p = reinterpret_cast<const char *>(base) + byte_offset;
+    if constexpr (sizeof(T) == 16)
+        return __builtin_bit_cast(T, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p)));
+    else
+        return __builtin_nontemporal_load(reinterpret_cast<const T *>(p));
 }
 
 __device__ __forceinline__ void st_at(float *base, uint32_t byte_offset, float v) {
     *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + byte_offset) = v;
+}
+
+// A uniform value, required in scalar registers where this is written: the load behind it is issued and
+// waited for here rather than where the value is first used.  The value itself is not redefined (an asm
+// output would hide from the compiler that a pointer is a kernel argument, i.e. global memory).
+template <class T>
+__device__ __forceinline__ T pin_s(T v) {
+    asm volatile("" ::"s"(v));
+    return v;
+}
+
+// The operands of one matrix of a launch, in scalar registers.
+struct MatOps {
+    const uint4 *qweight;
+    const int32_t *qzeros;
+    const float *scales;
+    const float *x;
+    const float *wn;
+    float *y;
+    int out;
+};
+
+__device__ __forceinline__ MatOps mat_ops(const Q4Mat &M) {
+    MatOps o;
+    o.qweight = pin_s(M.qweight);
+    o.qzeros = pin_s(M.qzeros);
+    o.scales = pin_s(M.scales);
+    o.x = pin_s(M.x);
+    o.wn = pin_s(M.wn);
+    o.y = pin_s(M.y);
+    o.out = pin_s(M.out);
+    return o;
 }
 
 struct RowData {
@@ -154,28 +196,51 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     __shared__ float red[NW];
     __shared__ float part[2][TR][NM][PW];
 
-    const int in = L.in;
+    // Every scalar operand the prologue needs is asked for here, at once, and pinned in SGPRs: a kernel's
+    // arguments are cold in the scalar cache, a load that misses takes some 0.3 us, and loads the compiler
+    // places where their values are first used follow each other (the matrix of this block, then its
+    // pointers, then the row geometry: three round trips in front of the first weight load).
+    const int in = pin_s(L.in);
+    const int n_mats = pin_s(L.n_mats);
+    const int groups = pin_s(L.groups);
+    const int rows_per_block = pin_s(L.rows_per_block);
+    const float eps = pin_s(L.eps);
+    // epilogue operands, uniform for the block
+    const int epi_kind = pin_s(L.e.kind);
+    const int n_scatter = pin_s(L.e.n_scatter);
+    const float *__restrict__ res = pin_s(L.e.res);
+    const int32_t *__restrict__ sc_idx[3] = {pin_s(L.e.sc_idx[0]), pin_s(L.e.sc_idx[1]), pin_s(L.e.sc_idx[2])};
+    float *__restrict__ sc_out[3] = {pin_s(L.e.sc_out[0]), pin_s(L.e.sc_out[1]), pin_s(L.e.sc_out[2])};
+    MatOps mat[NM];
+    int rb = blockIdx.x;
+    if constexpr (PAIR) {
+        mat[0] = mat_ops(L.m[0]);
+        mat[1] = mat_ops(L.m[1]);
+    } else {
+        const MatOps m0 = mat_ops(L.m[0]), m1 = mat_ops(L.m[1]), m2 = mat_ops(L.m[2]);
+        const int rb0 = pin_s(L.m[0].row_blocks), rb1 = pin_s(L.m[1].row_blocks);
+        mat[0] = m0;
+        if (n_mats > 1 && rb >= rb0) {
+            rb -= rb0;
+            mat[0] = m1;
+            if (n_mats > 2 && rb >= rb1) {
+                rb -= rb1;
+                mat[0] = m2;
+            }
+        }
+    }
     const int C = in >> 5;
     const int xstride = C * kChunkPad + C;
 
-    int rb = blockIdx.x;
-    int mi = 0;
-    if (!PAIR) {
-        while (mi + 1 < L.n_mats && rb >= L.m[mi].row_blocks) {
-            rb -= L.m[mi].row_blocks;
-            mi++;
-        }
-    }
     const int b = blockIdx.y;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int kslice = wave % NWK;
     const int stream = wave / NWK;
-    const int n_out = L.m[mi].out;
-    const int groups = L.groups;
-    const int row0 = rb * L.rows_per_block;
-    const int row1 = min(row0 + L.rows_per_block, n_out);
+    const int n_out = mat[0].out;
+    const int row0 = rb * rows_per_block;
+    const int row1 = min(row0 + rows_per_block, n_out);
     const int c = kslice * 64 + lane; // this lane's chunk, for good
     const bool has_chunk = c < C;
 
@@ -191,9 +256,9 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     const int32_t *__restrict__ zq[NM];
 #pragma unroll
     for (int q = 0; q < NM; q++) {
-        wq[q] = L.m[mi + q].qweight;
-        sc[q] = L.m[mi + q].scales;
-        zq[q] = L.m[mi + q].qzeros;
+        wq[q] = mat[q].qweight;
+        sc[q] = mat[q].scales;
+        zq[q] = mat[q].qzeros;
     }
     auto fetch = [&](int i, RowData(&d)[NM]) {
         const int o = min(row0 + stream + i * S, last);
@@ -214,14 +279,18 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     if constexpr (DIRECT) {
         // this wave's 64 chunks of x, 1 KB per load instruction (whole cache lines); past the end the last
         // 16 bytes are re-read and zeroed below
-        const float4 *xp = reinterpret_cast<const float4 *>(L.m[mi].x + (size_t)b * in);
+        const float4 *xp = reinterpret_cast<const float4 *>(mat[0].x + (size_t)b * in);
         const int n4 = in >> 2;
 #pragma unroll
         for (int i = 0; i < 8; i++) xd[i] = xp[min(kslice * 512 + i * 64 + lane, n4 - 1)];
     } else {
 #pragma unroll
         for (int q = 0; q < NM; q++)
-            stage_issue<NW>(L.m[mi + q].x + (size_t)b * in, L.m[mi + q].wn, in, 0, tid, xr[q]);
+            stage_issue<NW>(mat[q].x + (size_t)b * in, mat[q].wn, in, 0, tid, xr[q]);
+        // No wave of the block asks for weights before every wave has asked for its piece of x: a CU returns
+        // loads in the order it received them, and a piece of x (a cache hit) requested behind another wave's
+        // first rows (HBM) would hold up the staging of the whole block until those rows are in.
+        if constexpr (NW > 1) __builtin_amdgcn_s_barrier();
     }
     __builtin_amdgcn_sched_barrier(0);
     RowData pipe[P][NM];
@@ -235,7 +304,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     float sx[NM];     // fp32 form: sum of the chunk's x; integer form: sum of its q
     float xdelta[NM]; // integer form: the chunk's step
     float ss = 1.0f;
-    const bool norm = !DIRECT && L.m[mi].wn != nullptr;
+    const bool norm = !DIRECT && mat[0].wn != nullptr;
     if constexpr (DIRECT) {
         // Turned through a region of LDS of the wave's own, from "lane l holds floats 4l..4l+3 of every 256"
         // to "lane l holds its chunk's 32": no block barrier (a wave's LDS accesses execute in order).
@@ -264,7 +333,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         float ssq = 0.f;
 #pragma unroll
         for (int q = 0; q < NM; q++) {
-            const Q4Mat &M = L.m[mi + q];
+            const MatOps &M = mat[q];
             float *xs = lds + q * xstride;
             float p = stage_consume<NW>(M.wn != nullptr, in, 0, tid, xr[q], xs, xs + C * kChunkPad, 0.f);
             p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
@@ -280,7 +349,7 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
 #pragma unroll
             for (int i = 0; i < NW; i++) t += red[i];
             t /= (float)in;
-            t += L.eps;
+            t += eps;
             ss = 1.0f / sqrtf(t);
         }
         if constexpr (IDOT) {
@@ -341,15 +410,8 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     // the steady state alone: vmcnt leaves the P - 1 younger rows in flight.
     // Otherwise the issue order of the prologue leaks into the loop's waits.
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0), expcnt and lgkmcnt untouched
-    // Epilogue operands, uniform for the block.
-    const Q4Epi &E = L.e;
-    const int epi_kind = E.kind;
-    const int n_scatter = E.n_scatter;
     const size_t out_base = (size_t)b * n_out;
-    const float *__restrict__ res = E.res;
-    float *__restrict__ const yout = L.m[mi].y;
-    const int32_t *__restrict__ sc_idx[3] = {E.sc_idx[0], E.sc_idx[1], E.sc_idx[2]};
-    float *__restrict__ sc_out[3] = {E.sc_out[0], E.sc_out[1], E.sc_out[2]};
+    float *__restrict__ const yout = mat[0].y;
     // what the epilogue lanes prefetch; the scales (at least one word per row) stand in for absent operands
     const bool has_res = !PAIR && epi_kind == Q4_EPI_RESIDUAL;
     const float *__restrict__ res_p = has_res ? res + out_base : sc[0];
@@ -560,7 +622,7 @@ int launch_sg(Q4Launch &L, hipStream_t stream) {
             case 3: // 5120: 20 rows per block are one tile of 5 streams, 60 or so are four tiles either way
                 if (plan_cost(L, 3, 5, 4, false) < plan_cost(L, 3, 4, 4, false)) return launch_s<G, 3, 5, false, MODE>(L, stream);
                 return launch_s<G, 3, 4, false, MODE>(L, stream);
-            case 4: return launch_s<G, 4, 4, false, MODE>(L, stream);
+            case 4: return launch_s<G, 4, 4, false, MODE, 2>(L, stream); // 8192: rows of 4 KB; two in flight per stream measured faster than four (q|k|v 13.4 -> 12.2 us, wo 12.1 -> 10.9)
             case 5: case 6: return launch_s<G, 6, 2, false, MODE>(L, stream);
             case 7: return launch_s<G, 7, 2, false, MODE, 5>(L, stream); // 13824 -> 5120: 20 rows per block in two tiles
             case 8: return launch_s<G, 8, 2, false, MODE>(L, stream);
