@@ -13,6 +13,9 @@
 // adds a relative error of about |s - m| * 6e-8 to a weight).
 //
 // Compiled with -ffp-contract=off; FMAs appear only where written as fmaf().
+#include <stdlib.h>
+#include <string.h>
+
 #include "l2_internal.h"
 
 namespace {
@@ -362,6 +365,272 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
             if (d == 0) {
                 p[HS] = M;
                 p[HS + 1] = den;
+            }
+        }
+    }
+}
+
+// The same decode step for grouped-query models (4 or 8 query heads per kv head) on the matrix cores, all in
+// fp32 (v_mfma_f32_16x16x4_f32): the query heads of the kv head are columns of the tile, so a cache row
+// costs the same whatever their number, and the dot products need no cross-lane sums.
+//
+// A wave takes tiles of 16 timesteps.  With lane = (i = lane % 16, kb = lane / 16):
+//   S^T = K Q^T      A: lane (timestep i, kb) holds K[t][16 m + 4 kb + e], B: lane (head i, kb) holds
+//                    Q[head][16 m + 4 kb + e]; MFMA step (m, e), m < 8, e < 4, contracts over those four d.
+//                    The A operand is what a 16-byte load of the cache row gives: no LDS on the way.
+//   C layout         lane (head j, kb), register r -> timestep 4 kb + r: the four lanes of a head hold its
+//                    16 scores, the running maximum is shared by them, the running sum is per lane.
+//   O^T += V^T P^T   MFMA step (r, c) contracts over timesteps 4 kb + r, the lane's own register r of P: the
+//                    B operand needs no data movement.  A: lane (i, kb) holds V[4 kb + r][d] with
+//                    d = 64 (c / 4) + 4 i + c % 4, again a 16-byte load as it stands.  The accumulator c,
+//                    register r of lane (head j, kb) is O[head][64 (c / 4) + 16 kb + 4 r + c % 4].
+// Two tiles per wave are in flight (all their loads issued before any arithmetic); the four waves of a block
+// merge through LDS, the splits through attn_combine_kernel, as in the kernel above.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int QG>
+__global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(const AttnDecode A) {
+    constexpr int NWV = 4, NT = 256, TK = 16;
+    constexpr int HS = 128, HALF = 64;
+    static_assert(QG == 4 || QG == 8, "the query heads of a kv head fill part of the 16 columns of a tile");
+    __shared__ float qs[QG * HS];
+    __shared__ float kvnew[2][HS];
+    __shared__ float comb[NWV][QG][HS + 2];
+    const int kvh = blockIdx.x, sp = blockIdx.y;
+    const int pos = A.dpos ? A.dpos[0] : A.pos;
+    const int t0 = sp * A.ts;
+    if (t0 > pos) return;
+    const int t1 = min(t0 + A.ts, pos + 1);
+    const int n = t1 - t0;
+    const int kv_dim = A.n_kv_heads * HS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, kb = lane >> 4;
+
+    const float *__restrict__ kc = A.kcache;
+    const float *__restrict__ vc = A.vcache;
+    const uint32_t row_bytes = (uint32_t)kv_dim * 4u;
+    const int t_last = t1 - 1;
+    const uint32_t k_lane = (uint32_t)(kvh * HS + 4 * kb) * 4u; // + 64 m bytes
+    const uint32_t v_lane = (uint32_t)(kvh * HS + 4 * li) * 4u; // + 256 bytes for the second half of d
+
+    struct Tile {
+        float4 k[8]; // k[m]: K[t = li][16 m + 4 kb ..]
+        float4 v[8]; // v[2 r + half]: V[t = 4 kb + r][64 half + 4 li ..]
+    };
+    // Unconditional loads: rows past the end re-read the last row (masked below).
+    auto fetch = [&](int tile, Tile &d) {
+        const int tb = t0 + tile * TK;
+        const uint32_t ko = __umul24(min(tb + li, t_last), row_bytes) + k_lane;
+#pragma unroll
+        for (int m = 0; m < 8; m++) d.k[m] = ld_at<float4>(kc, ko + 64u * m);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint32_t vo = __umul24(min(tb + 4 * kb + r, t_last), row_bytes) + v_lane;
+            d.v[2 * r] = ld_at<float4>(vc, vo);
+            d.v[2 * r + 1] = ld_at<float4>(vc, vo + 256u);
+        }
+    };
+    // The small loads that the staging needs go out first (loads return in order).
+    const float *ct = A.cos_t + (size_t)pos * HALF;
+    const float *st = A.sin_t + (size_t)pos * HALF;
+    constexpr int NQ = (QG * HALF + NT - 1) / NT;
+    float qa[NQ], qb[NQ], qc[NQ], qsn[NQ];
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const int idx = (tid + r * NT) % (QG * HALF);
+        const int j = idx >> 6, i = idx & 63;
+        const float *qh = A.q + (size_t)(kvh * QG + j) * HS;
+        qa[r] = qh[i], qb[r] = qh[i + HALF];
+        qc[r] = ct[i], qsn[r] = st[i];
+    }
+    // where this thread's outputs go when the step is not split: fetched now, used at the very end
+    int sdst[QG * HS / NT];
+#pragma unroll
+    for (int u = 0; u < QG * HS / NT; u++) {
+        const int i = kvh * QG * HS + tid + u * NT;
+        sdst[u] = (A.scatter && A.n_splits == 1) ? A.scatter[i] : i;
+    }
+    const int hd = tid & 63;
+    const float nk_a = A.k_new[(size_t)kvh * HS + hd], nk_b = A.k_new[(size_t)kvh * HS + hd + HALF];
+    const float nv = A.v_new[(size_t)kvh * HS + (tid & 127)];
+    const float nc = ct[hd], ns = st[hd];
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int n_tiles = (n + TK - 1) / TK;
+    Tile ta, tb2;
+    fetch(wave, ta);
+    fetch(wave + NWV, tb2);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // q with RoPE, src/models.rs:100-129 (the second half uses the rotated first half)
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const int idx = (tid + r * NT) % (QG * HALF);
+        const int j = idx >> 6, i = idx & 63;
+        const float first = qa[r] * qc[r] - qb[r] * qsn[r];
+        qs[j * HS + i] = first;
+        qs[j * HS + HALF + i] = qb[r] * qc[r] + first * qsn[r];
+    }
+    // the new key, rotated, and the new value; the block whose range ends at pos also writes them to the
+    // cache (:236-249)
+    const bool owns_new = (t1 == pos + 1);
+    {
+        const float first = nk_a * nc - nk_b * ns;
+        const float second = nk_b * nc + first * ns;
+        kvnew[0][hd] = first;
+        kvnew[0][hd + HALF] = second;
+        kvnew[1][tid & 127] = nv;
+        if (owns_new) {
+            if (tid < HALF) {
+                float *kw = A.kcache + (size_t)pos * kv_dim + kvh * HS;
+                kw[tid] = first;
+                kw[tid + HALF] = second;
+            } else if (tid >= 128 && tid < 256) {
+                A.vcache[(size_t)pos * kv_dim + kvh * HS + (tid - 128)] = nv;
+            }
+        }
+    }
+    __syncthreads();
+
+    // B operands of the score MFMAs: this lane's head (columns beyond the QG heads are zero)
+    float4 qf[8];
+#pragma unroll
+    for (int m = 0; m < 8; m++)
+        qf[m] = li < QG ? *reinterpret_cast<const float4 *>(&qs[li * HS + 16 * m + 4 * kb]) : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    float m_run = kNoScore, l = 0.f;
+    v4f acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc[c] = v4f{0.f, 0.f, 0.f, 0.f};
+    // log2(e) / sqrt(head_size): src/models.rs:154 divides the score by sqrt(head_size)
+    const float scale = 1.44269504088896340736f / sqrtf((float)HS);
+
+    auto tile_math = [&](int tile, Tile &d) __attribute__((always_inline)) {
+        const int tb = t0 + tile * TK;
+        if (tb <= pos && pos < tb + TK) { // once per step: the row of the new position comes from LDS, not from the cache
+            if (tb + li == pos) {
+#pragma unroll
+                for (int m = 0; m < 8; m++) d.k[m] = *reinterpret_cast<const float4 *>(&kvnew[0][16 * m + 4 * kb]);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (tb + 4 * kb + r == pos) {
+                    d.v[2 * r] = *reinterpret_cast<const float4 *>(&kvnew[1][4 * li]);
+                    d.v[2 * r + 1] = *reinterpret_cast<const float4 *>(&kvnew[1][HALF + 4 * li]);
+                }
+        }
+        // scores: two accumulators, so that consecutive MFMAs do not wait for each other
+        v4f s0 = v4f{0.f, 0.f, 0.f, 0.f}, s1 = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < 8; m += 2) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].x, qf[m].x, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].x, qf[m + 1].x, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].y, qf[m].y, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].y, qf[m + 1].y, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].z, qf[m].z, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].z, qf[m + 1].z, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].w, qf[m].w, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].w, qf[m + 1].w, s1, 0, 0, 0);
+        }
+        float sc[4], p[4];
+        float mx = kNoScore;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const bool valid = tb + 4 * kb + r <= t_last;
+            sc[r] = valid ? (s0[r] + s1[r]) * scale : kNoScore;
+            mx = fmaxf(mx, sc[r]);
+        }
+        if (__any(mx > m_run)) { // some head's maximum moves: agree on it among the head's four lanes, rescale
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            const float c = exp2_fast(m_run - m_new);
+            l *= c;
+#pragma unroll
+            for (int cc = 0; cc < 8; cc++) acc[cc] *= c;
+            m_run = m_new;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const bool valid = tb + 4 * kb + r <= t_last;
+            p[r] = valid ? exp2_fast(sc[r] - m_run) : 0.f;
+            l += p[r];
+        }
+        // weighted sums: eight independent accumulators
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float4 v0 = d.v[2 * r], v1 = d.v[2 * r + 1];
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.x, p[r], acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.y, p[r], acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.z, p[r], acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.w, p[r], acc[3], 0, 0, 0);
+            acc[4] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.x, p[r], acc[4], 0, 0, 0);
+            acc[5] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.y, p[r], acc[5], 0, 0, 0);
+            acc[6] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.z, p[r], acc[6], 0, 0, 0);
+            acc[7] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.w, p[r], acc[7], 0, 0, 0);
+        }
+    };
+    // Tiles wave, wave + 4, ...: two buffers, each refilled right after its tile is done when the wave has a
+    // further tile for it (a uniform branch; up to two tiles per wave, the usual case behind a long cache,
+    // nothing is refilled).
+    for (int tile = wave; tile < n_tiles; tile += 2 * NWV) {
+        tile_math(tile, ta);
+        if (tile + 2 * NWV < n_tiles) fetch(tile + 2 * NWV, ta);
+        if (tile + NWV < n_tiles) {
+            tile_math(tile + NWV, tb2);
+            if (tile + 3 * NWV < n_tiles) fetch(tile + 3 * NWV, tb2);
+        }
+    }
+
+    // this wave's (m, l, O) -> LDS.  The head's four lanes hold disjoint d: lane (j, kb), accumulators 0..3,
+    // register r are d = 16 kb + 4 r + 0..3, accumulators 4..7 the same 64 further on.
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    if (li < QG) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            *reinterpret_cast<float4 *>(&comb[wave][li][16 * kb + 4 * r]) = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+            *reinterpret_cast<float4 *>(&comb[wave][li][HALF + 16 * kb + 4 * r]) =
+                make_float4(acc[4][r], acc[5][r], acc[6][r], acc[7][r]);
+        }
+        if (kb == 0) {
+            comb[wave][li][HS] = m_run;
+            comb[wave][li][HS + 1] = l;
+        }
+    }
+    __syncthreads();
+    // merge the four waves; one thread per (head, dim), the passes unrolled so that their LDS reads overlap
+    constexpr int NP = QG * HS / NT;
+    float num[NP], den[NP], Mx[NP];
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+        const int idx = tid + u * NT;
+        const int j = idx >> 7, d = idx & 127;
+        float M = comb[0][j][HS];
+#pragma unroll
+        for (int w = 1; w < NWV; w++) M = fmaxf(M, comb[w][j][HS]);
+        float nu = 0.f, de = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWV; w++) {
+            const float e = exp2_fast(comb[w][j][HS] - M);
+            nu = fmaf(e, comb[w][j][d], nu);
+            de = fmaf(e, comb[w][j][HS + 1], de);
+        }
+        num[u] = nu, den[u] = de, Mx[u] = M;
+    }
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+        const int idx = tid + u * NT;
+        const int j = idx >> 7, d = idx & 127;
+        const int h = kvh * QG + j;
+        if (A.n_splits == 1) {
+            A.out[sdst[u]] = num[u] / den[u];
+        } else {
+            float *pp = A.part + ((size_t)h * A.max_splits + sp) * (HS + 2);
+            pp[d] = num[u];
+            if (d == 0) {
+                pp[HS] = Mx[u];
+                pp[HS + 1] = den[u];
             }
         }
     }
@@ -797,6 +1066,17 @@ __global__ __launch_bounds__(512) void attn_combine_kernel(const AttnDecode A) {
 
 template <int QG>
 int attn_launch_qg(const AttnDecode &a, hipStream_t st) {
+    if constexpr (QG >= 4) {
+        static const bool valu = []() {
+            const char *v = getenv("L2_ATTN_IMPL");
+            return v && !strcmp(v, "valu");
+        }();
+        if (!valu) {
+            hipLaunchKernelGGL((attn_decode_mfma_kernel<QG>), dim3(a.n_kv_heads, a.n_splits), dim3(256), 0, st, a);
+            L2_HIP(hipGetLastError());
+            return L2_OK;
+        }
+    }
     constexpr size_t lds = QG >= 4 ? (size_t)16 * QG * 130 * sizeof(float) : 0; // the partial results of 16 rows
     if (lds > 48 * 1024) {
         static bool raised = false; // per instantiation
