@@ -235,7 +235,9 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     const int b = blockIdx.y;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // the wave's number as a scalar: the row a wave works on, and with it the row's part of every address and
+    // the shift that extracts its zero point, are then scalar arithmetic, off the vector ALU
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kslice = wave % NWK;
     const int stream = wave / NWK;
     const int n_out = mat[0].out;
@@ -260,15 +262,14 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         sc[q] = mat[q].scales;
         zq[q] = mat[q].qzeros;
     }
+    const uint32_t cc16 = (uint32_t)cc << 4, g4 = (uint32_t)g << 2; // the lane's part of the byte offsets
     auto fetch = [&](int i, RowData(&d)[NM]) {
-        const int o = min(row0 + stream + i * S, last);
+        const int o = min(row0 + stream + i * S, last); // uniform: the row's part of an address is scalar work
 #pragma unroll
         for (int q = 0; q < NM; q++) {
-            // 24-bit multiplies and 32-bit byte offsets from a uniform base:
-            // no 64-bit address arithmetic per load
-            d[q].w = ld_at<uint4>(wq[q], (__umul24(o, C) + cc) << 4);
-            d[q].s = ld_at<float>(sc[q], (__umul24(o, groups) + g) << 2);
-            d[q].z = ld_at<int32_t>(zq[q], (__umul24(o >> 3, groups) + g) << 2);
+            d[q].w = ld_at<uint4>(reinterpret_cast<const char *>(wq[q]) + ((uint32_t)(o * C) << 4), cc16);
+            d[q].s = ld_at<float>(reinterpret_cast<const char *>(sc[q]) + ((uint32_t)(o * groups) << 2), g4);
+            d[q].z = ld_at<int32_t>(reinterpret_cast<const char *>(zq[q]) + ((uint32_t)((o >> 3) * groups) << 2), g4);
         }
     };
 
@@ -398,6 +399,9 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         }
     }
 
+    float nsx[NM];
+#pragma unroll
+    for (int q = 0; q < NM; q++) nsx[q] = -sx[q];
     const int n_rows = row1 - row0;
     // Steps of the longest stream; whole tiles of P steps run in the loop, what is left runs once after it,
     // straight-line and without refills, so that the loop body stays one block (and its waits exact).
@@ -423,14 +427,14 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     auto row_dot = [&](int o, const RowData(&d)[NM], float(&pr)[NM]) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < NM; q++) {
-            const int zn = (d[q].z >> (4 * (o & 7))) & 15;
+            const int zn = (int)(((uint32_t)d[q].z >> (4 * (o & 7))) & 15u);
             if constexpr (IDOT) {
                 const float f = chunk_idot(d[q].w, xp[q]);
                 pr[q] = (d[q].s * xdelta[q]) * fmaf(-(float)(zn - 7), sx[q], f);
             } else {
                 const float p = chunk_dot(d[q].w, x[q]);
-                const float z1 = (float)(zn + 1);
-                pr[q] = d[q].s * fmaf(p, 512.0f, -z1 * sx[q]);
+                // -(zn + 1) sx as one FMA on the converted nibble (the same real number, rounded once either way)
+                pr[q] = d[q].s * fmaf(p, 512.0f, fmaf((float)zn, nsx[q], nsx[q]));
             }
         }
     };
