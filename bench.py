@@ -236,11 +236,14 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool) -
         m.reset()
         m.forward(prompt[:min(chunk, n)], np.arange(min(chunk, n), dtype=np.int32))  # warm-up chunk
         m.reset()
+        toks = np.concatenate([[1], prompt[:n - 1]]).astype(np.int32)  # START-shifted, as prefill<A> does
         t0 = time.perf_counter()
-        for c0 in range(0, n, chunk):
-            c1 = min(c0 + chunk, n)
-            toks = np.concatenate([[1], prompt[:c1 - 1]])[c0:c1].astype(np.int32)  # START-shifted, as prefill<A> does
-            m.forward(toks, np.arange(c0, c1, dtype=np.int32))
+        if os.environ.get("L2_BENCH_PREFILL") == "serial":   # chunk by chunk through transformer<B>
+            for c0 in range(0, n, chunk):
+                c1 = min(c0 + chunk, n)
+                m.forward(toks[c0:c1], np.arange(c0, c1, dtype=np.int32))
+        else:
+            m.prefill_chunks(toks, 0, chunk)
         return time.perf_counter() - t0
 
     t_mfma = run(_lib.PREFILL_MFMA)

@@ -189,6 +189,13 @@ int l2_model_classifier(l2_model *m, const float *x_host, float *y_host);
 int l2_forward(l2_model *m, l2_state *s, const int32_t *tokens, const int32_t *pos, int B,
                float *logits_host);
 
+/* prefill::<A> over a whole prompt (src/inference.rs:16-40, the calls at :78-127 with one A): tokens[i], host
+ * i32[n], goes to position pos0 + i; the prompt is cut into chunks of `chunk` tokens (the last one may be
+ * shorter) and every chunk is what l2_forward computes for it, cache rows included; no logits.  In the
+ * matrix-core mode consecutive chunks run on two HIP streams of the model, one layer apart (a chunk needs from
+ * the one before it only that chunk's cache rows of the same layer); the call returns when all are done. */
+int l2_prefill_chunks(l2_model *m, l2_state *s, const int32_t *tokens, int n, int pos0, int chunk);
+
 /* One iteration of the B=1 loop at temperature 0 (src/inference.rs:141-162):
  * forward, then util::argmax (src/util.rs:39-46, ties -> last index) on the
  * device.  Only the token id crosses the boundary. */

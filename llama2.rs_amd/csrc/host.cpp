@@ -300,6 +300,22 @@ struct l2_model {
     size_t gemm_ws_floats = 0;
     int32_t *dtok = nullptr, *dpos = nullptr;
     unsigned long long *amax = nullptr;
+    // l2_prefill_chunks: a second stream with a second set of chunk buffers (consecutive chunks of a prompt run
+    // side by side, one layer apart), the whole prompt's ids and positions, one event per layer and stream
+    hipStream_t stream2 = nullptr;
+    struct ChunkBufs {
+        float *x = nullptr, *xq = nullptr, *xk = nullptr, *xv = nullptr, *qv = nullptr, *kv = nullptr, *vv = nullptr;
+        void *h16a = nullptr, *h16b = nullptr, *h16c = nullptr;
+        float *hb = nullptr, *hb2 = nullptr, *ssb = nullptr, *gemm_ws = nullptr;
+        size_t gemm_ws_floats = 0;
+        const int32_t *dtok = nullptr, *dpos = nullptr;
+    };
+    ChunkBufs alt;
+    int cap_B_alt = 0;
+    int32_t *pf_tok = nullptr, *pf_pos = nullptr;
+    int cap_pf = 0;
+    std::vector<hipEvent_t> pf_ev[2];
+    hipEvent_t pf_join = nullptr;
     int32_t *dprompt = nullptr, *dout_ids = nullptr;
     int cap_prompt = 0, cap_out = 0;
     // The decode step as a HIP graph (one per bucket of positions, kept in the state).  Off by default: a
@@ -669,6 +685,14 @@ extern "C" void l2_model_close(l2_model *m) {
                     m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y, m->h16a, m->h16b, m->h16c,
                     m->hb, m->hb2, m->ssb, m->gemm_ws};
     for (void *p : ptrs) dfree(p);
+    if (m->stream2) (void)hipStreamSynchronize(m->stream2);
+    void *alts[] = {m->alt.x, m->alt.xq, m->alt.xk, m->alt.xv, m->alt.qv, m->alt.kv, m->alt.vv, m->alt.h16a, m->alt.h16b,
+                    m->alt.h16c, m->alt.hb, m->alt.hb2, m->alt.ssb, m->alt.gemm_ws, m->pf_tok, m->pf_pos};
+    for (void *p : alts) dfree(p);
+    for (auto &v : m->pf_ev)
+        for (hipEvent_t e : v) (void)hipEventDestroy(e);
+    if (m->pf_join) (void)hipEventDestroy(m->pf_join);
+    if (m->stream2) (void)hipStreamDestroy(m->stream2);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
@@ -1280,25 +1304,37 @@ static int ensure_batch_mfma(l2_model *m, int B) {
 // with every QLinear as a dequant -> fp16 -> MFMA GEMM over the B tokens and the
 // element-wise steps as kernels of their own.  Logits are never produced here
 // (src/models.rs:288).
-static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
+static l2_model::ChunkBufs primary_bufs(const l2_model *m) {
+    l2_model::ChunkBufs b;
+    b.x = m->x, b.xq = m->xq, b.xk = m->xk, b.xv = m->xv, b.qv = m->qv, b.kv = m->kv, b.vv = m->vv;
+    b.h16a = m->h16a, b.h16b = m->h16b, b.h16c = m->h16c;
+    b.hb = m->hb, b.hb2 = m->hb2, b.ssb = m->ssb, b.gemm_ws = m->gemm_ws, b.gemm_ws_floats = m->gemm_ws_floats;
+    b.dtok = m->dtok, b.dpos = m->dpos;
+    return b;
+}
+
+// The chunk's buffers and stream are arguments: l2_prefill_chunks runs consecutive chunks on two streams.  What a
+// chunk needs from the one before it is that chunk's cache rows of the same layer, so `after_kv[l]` is recorded
+// behind the kernel that writes this chunk's rows of layer l and `before_attn[l]` is waited for in front of the
+// attention of layer l (either may be null).
+static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos, const l2_model::ChunkBufs &b,
+                                hipStream_t st, const hipEvent_t *after_kv, const hipEvent_t *before_attn) {
     L2_TRY(check_position(m, max_pos));
     const l2_dims &d = m->d;
     const int dim = d.dim, hid = d.hidden_dim, kvd = m->kv_dim, L = d.n_layers;
-    hipStream_t st = m->stream;
-    L2_TRY(ensure_batch_mfma(m, B));
     {
         ScatterTargets t{};
         t.n = 3;
         t.inv[0] = m->q[L2_WQ][0].inv_index, t.inv[1] = m->q[L2_WK][0].inv_index, t.inv[2] = m->q[L2_WV][0].inv_index;
-        t.out[0] = m->xq, t.out[1] = m->xk, t.out[2] = m->xv;
-        L2_TRY(embed_launch(m->x, m->tok_emb, m->dtok, dim, B, t, m->amax, st));
+        t.out[0] = b.xq, t.out[1] = b.xk, t.out[2] = b.xv;
+        L2_TRY(embed_launch(b.x, m->tok_emb, b.dtok, dim, B, t, nullptr, st));
         // the first layer's inputs; every later layer gets them from the kernel that ends the layer before
-        L2_TRY(rms_scale_launch(m->ssb, m->x, m->rms_eps, dim, B, st));
+        L2_TRY(rms_scale_launch(b.ssb, b.x, m->rms_eps, dim, B, st));
         PrepList P{};
         P.n_mats = 3;
-        P.out[0] = m->h16a, P.x[0] = m->xq, P.wn[0] = m->dwn + 0 * (size_t)dim;
-        P.out[1] = m->h16b, P.x[1] = m->xk, P.wn[1] = m->dwn + 1 * (size_t)dim;
-        P.out[2] = m->h16c, P.x[2] = m->xv, P.wn[2] = m->dwn + 2 * (size_t)dim;
+        P.out[0] = b.h16a, P.x[0] = b.xq, P.wn[0] = m->dwn + 0 * (size_t)dim;
+        P.out[1] = b.h16b, P.x[1] = b.xk, P.wn[1] = m->dwn + 1 * (size_t)dim;
+        P.out[2] = b.h16c, P.x[2] = b.xv, P.wn[2] = m->dwn + 2 * (size_t)dim;
         L2_TRY(prep_f16_multi_launch(P, dim, B, st));
     }
     for (int l = 0; l < L; l++) {
@@ -1308,63 +1344,70 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
         RopeKvArgs R{};
         {
             Q4Launch Q = launch_of(wq, B, m->rms_eps);
-            Q.m[0] = mat_of(wq, nullptr, nullptr, m->qv);
-            Q.m[1] = mat_of(wk, nullptr, nullptr, m->kv);
-            Q.m[2] = mat_of(wv, nullptr, nullptr, m->vv);
+            Q.m[0] = mat_of(wq, nullptr, nullptr, b.qv);
+            Q.m[1] = mat_of(wk, nullptr, nullptr, b.kv);
+            Q.m[2] = mat_of(wv, nullptr, nullptr, b.vv);
             Q.n_mats = 3;
-            XhList X{{m->h16a, m->h16b, m->h16c}};
+            XhList X{{b.h16a, b.h16b, b.h16c}};
             // partial tiles; the kernel that adds them also applies the rms scale, RoPE and the cache write
-            L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st, &R.KS));
+            L2_TRY(q4_gemm_launch(Q, X, b.ssb, b.gemm_ws, b.gemm_ws_floats, st, &R.KS));
         }
         float *kc = s->kcache + (size_t)l * m->max_seq * kvd;
         float *vc = s->vcache + (size_t)l * m->max_seq * kvd;
-        R.ws = m->gemm_ws, R.B = B, R.ss = m->ssb, R.pos = m->dpos, R.cos_t = m->rope_cos, R.sin_t = m->rope_sin;
-        R.q = m->qv, R.kcache = kc, R.vcache = vc, R.n_heads = d.n_heads, R.n_kv_heads = d.n_kv_heads;
+        R.ws = b.gemm_ws, R.B = B, R.ss = b.ssb, R.pos = b.dpos, R.cos_t = m->rope_cos, R.sin_t = m->rope_sin;
+        R.q = b.qv, R.kcache = kc, R.vcache = vc, R.n_heads = d.n_heads, R.n_kv_heads = d.n_kv_heads;
         L2_TRY(gemm_rope_kv_launch(R, st));
-        L2_TRY(attention_launch(nullptr, m->h16a, m->qv, kc, vc, m->dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
+        if (after_kv) L2_HIP(hipEventRecord(after_kv[l], st));
+        if (before_attn) L2_HIP(hipStreamWaitEvent(st, before_attn[l], 0));
+        L2_TRY(attention_launch(nullptr, b.h16a, b.qv, kc, vc, b.dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
                                 m->head_size, max_pos, B, st));
         {   // wo: partial tiles, then residual + rms scale + the fp16 inputs of w1 and w3 in one kernel
             Q4Launch Q = launch_of(wo, B, 0.f);
-            Q.m[0] = mat_of(wo, nullptr, nullptr, m->x);
-            XhList X{{m->h16a, nullptr, nullptr}};
+            Q.m[0] = mat_of(wo, nullptr, nullptr, b.x);
+            XhList X{{b.h16a, nullptr, nullptr}};
             ResNormPrep R{};
-            L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st, &R.KS));
-            R.ws = m->gemm_ws, R.B = B, R.out = dim, R.res = m->x, R.x = m->x, R.ss = m->ssb, R.eps = m->rms_eps;
+            L2_TRY(q4_gemm_launch(Q, X, nullptr, b.gemm_ws, b.gemm_ws_floats, st, &R.KS));
+            R.ws = b.gemm_ws, R.B = B, R.out = dim, R.res = b.x, R.x = b.x, R.ss = b.ssb, R.eps = m->rms_eps;
             R.n = 2, R.wn = m->rms_ffn + (size_t)l * dim;
-            R.inv[0] = w1.inv_index, R.out_h[0] = m->h16a;
-            R.inv[1] = w3.inv_index, R.out_h[1] = m->h16b;
+            R.inv[0] = w1.inv_index, R.out_h[0] = b.h16a;
+            R.inv[1] = w3.inv_index, R.out_h[1] = b.h16b;
             L2_TRY(gemm_residual_norm_prep_launch(R, st));
         }
         {
             Q4Launch Q = launch_of(w1, B, m->rms_eps);
-            Q.m[0] = mat_of(w1, nullptr, nullptr, m->hb);
-            Q.m[1] = mat_of(w3, nullptr, nullptr, m->hb2);
+            Q.m[0] = mat_of(w1, nullptr, nullptr, b.hb);
+            Q.m[1] = mat_of(w3, nullptr, nullptr, b.hb2);
             Q.n_mats = 2;
-            XhList X{{m->h16a, m->h16b, nullptr}};
-            L2_TRY(q4_gemm_launch(Q, X, m->ssb, m->gemm_ws, m->gemm_ws_floats, st));
+            XhList X{{b.h16a, b.h16b, nullptr}};
+            L2_TRY(q4_gemm_launch(Q, X, b.ssb, b.gemm_ws, b.gemm_ws_floats, st));
         }
-        L2_TRY(silu_scatter_launch(nullptr, m->h16a, m->hb, m->hb2, w2.inv_index, hid, B, st));
+        L2_TRY(silu_scatter_launch(nullptr, b.h16a, b.hb, b.hb2, w2.inv_index, hid, B, st));
         {
             Q4Launch Q = launch_of(w2, B, 0.f);
-            Q.m[0] = mat_of(w2, nullptr, nullptr, m->x);
-            XhList X{{m->h16a, nullptr, nullptr}};
+            Q.m[0] = mat_of(w2, nullptr, nullptr, b.x);
+            XhList X{{b.h16a, nullptr, nullptr}};
             if (l + 1 < L) { // the same kernel hands the next layer its q, k and v inputs
                 ResNormPrep R{};
-                L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st, &R.KS));
-                R.ws = m->gemm_ws, R.B = B, R.out = dim, R.res = m->x, R.x = m->x, R.ss = m->ssb, R.eps = m->rms_eps;
+                L2_TRY(q4_gemm_launch(Q, X, nullptr, b.gemm_ws, b.gemm_ws_floats, st, &R.KS));
+                R.ws = b.gemm_ws, R.B = B, R.out = dim, R.res = b.x, R.x = b.x, R.ss = b.ssb, R.eps = m->rms_eps;
                 R.n = 3, R.wn = m->rms_att + (size_t)(l + 1) * dim;
-                R.inv[0] = m->q[L2_WQ][l + 1].inv_index, R.out_h[0] = m->h16a;
-                R.inv[1] = m->q[L2_WK][l + 1].inv_index, R.out_h[1] = m->h16b;
-                R.inv[2] = m->q[L2_WV][l + 1].inv_index, R.out_h[2] = m->h16c;
+                R.inv[0] = m->q[L2_WQ][l + 1].inv_index, R.out_h[0] = b.h16a;
+                R.inv[1] = m->q[L2_WK][l + 1].inv_index, R.out_h[1] = b.h16b;
+                R.inv[2] = m->q[L2_WV][l + 1].inv_index, R.out_h[2] = b.h16c;
                 L2_TRY(gemm_residual_norm_prep_launch(R, st));
             } else {
                 Q.e.kind = Q4_EPI_RESIDUAL;
-                Q.e.res = m->x;
-                L2_TRY(q4_gemm_launch(Q, X, nullptr, m->gemm_ws, m->gemm_ws_floats, st));
+                Q.e.res = b.x;
+                L2_TRY(q4_gemm_launch(Q, X, nullptr, b.gemm_ws, b.gemm_ws_floats, st));
             }
         }
     }
     return L2_OK;
+}
+
+static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos) {
+    L2_TRY(ensure_batch_mfma(m, B));
+    return forward_enqueue_mfma(m, s, B, max_pos, primary_bufs(m), m->stream, nullptr, nullptr);
 }
 
 static int check_tokens(const l2_model *m, const int32_t *tokens, const int32_t *pos, int B, int *max_pos) {
@@ -1396,6 +1439,114 @@ extern "C" int l2_forward(l2_model *m, l2_state *s, const int32_t *tokens, const
         L2_TRY(forward_enqueue(m, s, B, max_pos, B == 1));
     if (B == 1 && logits_host)
         L2_HIP(hipMemcpyAsync(logits_host, m->logits, (size_t)m->d.vocab_size * 4, hipMemcpyDeviceToHost, m->stream));
+    L2_HIP(hipStreamSynchronize(m->stream));
+    return L2_OK;
+}
+
+// The second set of chunk buffers, the second stream and the per-layer events of l2_prefill_chunks.
+static int ensure_prefill_pipeline(l2_model *m, int B, int n) {
+    if (!m->stream2) L2_HIP(hipStreamCreate(&m->stream2)); // default priority, as the model's own
+    if (!m->pf_join) L2_HIP(hipEventCreateWithFlags(&m->pf_join, hipEventDisableTiming));
+    for (auto &v : m->pf_ev)
+        while ((int)v.size() < m->d.n_layers) {
+            hipEvent_t e = nullptr;
+            L2_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            v.push_back(e);
+        }
+    if (n > m->cap_pf) {
+        L2_HIP(hipStreamSynchronize(m->stream));
+        L2_HIP(hipStreamSynchronize(m->stream2));
+        dfree(m->pf_tok), dfree(m->pf_pos);
+        m->pf_tok = m->pf_pos = nullptr, m->cap_pf = 0;
+        L2_TRY(dalloc(&m->pf_tok, (size_t)n));
+        L2_TRY(dalloc(&m->pf_pos, (size_t)n));
+        m->cap_pf = n;
+    }
+    if (B <= m->cap_B_alt) return L2_OK;
+    L2_HIP(hipStreamSynchronize(m->stream2));
+    l2_model::ChunkBufs &a = m->alt;
+    void **bufs[] = {(void **)&a.x, (void **)&a.xq, (void **)&a.xk, (void **)&a.xv, (void **)&a.qv, (void **)&a.kv,
+                     (void **)&a.vv, &a.h16a, &a.h16b, &a.h16c, (void **)&a.hb, (void **)&a.hb2, (void **)&a.ssb,
+                     (void **)&a.gemm_ws};
+    for (void **b : bufs) {
+        dfree(*b);
+        *b = nullptr;
+    }
+    m->cap_B_alt = 0;
+    const size_t dim = m->d.dim, hid = m->d.hidden_dim, kvd = m->kv_dim, wide = std::max(dim, hid);
+    L2_TRY(dalloc(&a.x, B * dim));
+    L2_TRY(dalloc(&a.xq, B * dim));
+    L2_TRY(dalloc(&a.xk, B * dim));
+    L2_TRY(dalloc(&a.xv, B * dim));
+    L2_TRY(dalloc(&a.qv, B * dim));
+    L2_TRY(dalloc(&a.kv, B * kvd));
+    L2_TRY(dalloc(&a.vv, B * kvd));
+    uint16_t *h = nullptr;
+    L2_TRY(dalloc(&h, B * wide));
+    a.h16a = h;
+    L2_TRY(dalloc(&h, B * wide));
+    a.h16b = h;
+    L2_TRY(dalloc(&h, B * wide));
+    a.h16c = h;
+    L2_TRY(dalloc(&a.hb, B * hid));
+    L2_TRY(dalloc(&a.hb2, B * hid));
+    L2_TRY(dalloc(&a.ssb, (size_t)B));
+    a.gemm_ws_floats = (size_t)8 * B * std::max((size_t)2 * hid, dim + 2 * kvd) / 2;
+    L2_TRY(dalloc(&a.gemm_ws, a.gemm_ws_floats));
+    m->cap_B_alt = B;
+    return L2_OK;
+}
+
+// prefill<A> (src/inference.rs:16-40) for a whole prompt: tokens[i] at position pos0 + i, in chunks of `chunk`,
+// no logits.  With the matrix-core mode consecutive chunks run on two streams, each with buffers of its own:
+// a chunk needs from its predecessor only that chunk's cache rows of the same layer (an event per layer), so
+// the second chunk follows one layer behind the first and its kernels fill the compute units that the first
+// one's short launches leave idle.  The arithmetic of a chunk is that of l2_forward on the same chunk.
+extern "C" int l2_prefill_chunks(l2_model *m, l2_state *s, const int32_t *tokens, int n, int pos0, int chunk) {
+    if (!m || !s || !tokens) return l2_fail(L2_ERR_ARG, "null argument");
+    if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
+    if (n < 1 || chunk < 1 || chunk > 4096) return l2_fail(L2_ERR_RANGE, "%d tokens in chunks of %d (1..4096)", n, chunk);
+    if (pos0 < 0 || (long)pos0 + n > m->max_seq)
+        return l2_fail(L2_ERR_RANGE, "positions %d..%ld outside 0..%d", pos0, (long)pos0 + n - 1, m->max_seq - 1);
+    for (int i = 0; i < n; i++)
+        if (tokens[i] < 0 || tokens[i] >= m->d.vocab_size)
+            return l2_fail(L2_ERR_RANGE, "token id %d outside 0..%d", tokens[i], m->d.vocab_size - 1);
+    const int Bmax = std::min(chunk, n);
+    L2_TRY(ensure_batch(m, Bmax));
+    const bool mfma = m->prefill_mode == L2_PREFILL_MFMA;
+    if (mfma) L2_TRY(ensure_batch_mfma(m, Bmax));
+    L2_TRY(ensure_prefill_pipeline(m, mfma ? Bmax : 0, n));
+    std::vector<int32_t> pos((size_t)n);
+    for (int i = 0; i < n; i++) pos[(size_t)i] = pos0 + i;
+    // synchronous copies: the host arrays are the caller's and this function's own
+    L2_HIP(hipStreamSynchronize(m->stream));
+    L2_HIP(hipMemcpy(m->pf_tok, tokens, (size_t)n * 4, hipMemcpyHostToDevice));
+    L2_HIP(hipMemcpy(m->pf_pos, pos.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    int c = 0;
+    for (int c0 = 0; c0 < n; c0 += chunk, c++) {
+        const int B = std::min(chunk, n - c0);
+        const int max_pos = pos0 + c0 + B - 1;
+        if (mfma && B > 1) {
+            l2_model::ChunkBufs b = (c & 1) ? m->alt : primary_bufs(m);
+            b.dtok = m->pf_tok + c0, b.dpos = m->pf_pos + c0;
+            hipStream_t st = (c & 1) ? m->stream2 : m->stream;
+            L2_TRY(forward_enqueue_mfma(m, s, B, max_pos, b, st, m->pf_ev[c & 1].data(),
+                                        c > 0 ? m->pf_ev[(c - 1) & 1].data() : nullptr));
+        } else {
+            // one token left over, or the fp32 mode: the fp32 kernels on the model's stream, behind everything
+            if (c > 0 && mfma) {
+                L2_HIP(hipEventRecord(m->pf_join, m->stream2));
+                L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+            }
+            L2_HIP(hipMemcpyAsync(m->dtok, m->pf_tok + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
+            L2_HIP(hipMemcpyAsync(m->dpos, m->pf_pos + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
+            L2_TRY(forward_enqueue(m, s, B, max_pos, false));
+        }
+    }
+    if (mfma) {
+        L2_HIP(hipEventRecord(m->pf_join, m->stream2));
+        L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+    }
     L2_HIP(hipStreamSynchronize(m->stream));
     return L2_OK;
 }

@@ -71,6 +71,7 @@ SIGNATURES = {
     "l2_model_qmatvec": (_I, [_VP, _I, _I, _VP, _I, _VP]),
     "l2_model_classifier": (_I, [_VP, _VP, _VP]),
     "l2_forward": (_I, [_VP, _VP, _VP, _VP, _I, _VP]),
+    "l2_prefill_chunks": (_I, [_VP, _VP, _VP, _I, _I, _I]),
     "l2_decode_greedy": (_I, [_VP, _VP, C.c_int32, C.c_int32, C.POINTER(C.c_int32)]),
     "l2_generate_greedy": (_I, [_VP, _VP, _VP, _I, _I, _I, _VP, C.POINTER(_I), C.POINTER(C.c_double)]),
     "l2_tokenizer_open": (_I, [C.c_char_p, _I, C.POINTER(_VP)]),

@@ -183,6 +183,11 @@ class Model:
                                _p(logits) if logits is not None else None))
         return logits
 
+    def prefill_chunks(self, tokens, pos0: int, chunk: int) -> None:
+        """prefill::<A> over a whole prompt: tokens[i] at position pos0 + i, in chunks of `chunk`."""
+        tokens = _i32(tokens)
+        check(lib().l2_prefill_chunks(self.h, self.state, _p(tokens), tokens.shape[0], pos0, chunk))
+
     def decode_greedy(self, token: int, pos: int) -> int:
         nxt = C.c_int32()
         check(lib().l2_decode_greedy(self.h, self.state, token, pos, C.byref(nxt)))

@@ -568,6 +568,50 @@ GQA8_G64 = ck.Dims(dim=1024, hidden_dim=1408, n_layers=2, n_heads=8, n_kv_heads=
                    seq_len=160, group_size=64)   # the 70B head geometry and group size, small
 
 
+@pytest.mark.parametrize("mode", ["mfma", "fp32"])
+@pytest.mark.parametrize("n,chunk", [(512, 128), (300, 128), (257, 64), (40, 64), (9, 2)],
+                         ids=["four_chunks", "short_last_chunk", "one_token_left", "one_short_chunk", "chunks_of_2"])
+def test_prefill_chunks_equals_chunk_by_chunk(ops, n, chunk, mode):
+    """prefill<A> over a whole prompt (src/inference.rs:16-40) through l2_prefill_chunks, whose chunks overlap on
+    two streams in the matrix-core mode, against the same chunks given to transformer<B> one by one: every cache
+    row of every layer and the logits that follow, bit for bit (the kernels and their operands are the same)."""
+    from llama2_rs import _lib
+    from llama2_rs._lib import L2Error
+    dims = ck.Dims(dim=512, hidden_dim=768, n_layers=3, n_heads=4, n_kv_heads=2, vocab_size=400, seq_len=n + 8,
+                   group_size=128)
+    img = ck.synth_weights_image(dims, seed=11)
+    m = ops.Model(img, dims)
+    m.set_prefill_mode(_lib.PREFILL_MFMA if mode == "mfma" else _lib.PREFILL_FP32)
+    rng = np.random.default_rng(n)
+    toks = rng.integers(0, dims.vocab_size, size=n).astype(np.int32)
+
+    def rows_and_logits():
+        rows = [m.read_kv(l, 0, n) for l in range(dims.n_layers)]
+        return rows, m.forward([5], [n])
+
+    for rep in range(2):    # the second pass reuses both sets of buffers and the events
+        m.reset()
+        for c0 in range(0, n, chunk):
+            c1 = min(c0 + chunk, n)
+            m.forward(toks[c0:c1], np.arange(c0, c1, dtype=np.int32))
+        want_rows, want_logits = rows_and_logits()
+        m.reset()
+        m.prefill_chunks(toks, 0, chunk)
+        got_rows, got_logits = rows_and_logits()
+        for l in range(dims.n_layers):
+            np.testing.assert_array_equal(got_rows[l][0], want_rows[l][0])
+            np.testing.assert_array_equal(got_rows[l][1], want_rows[l][1])
+        np.testing.assert_array_equal(got_logits, want_logits)
+    # arguments: a prompt that does not fit the cache, an id outside the vocabulary
+    with pytest.raises(L2Error):
+        m.prefill_chunks(toks, 9, chunk)
+    bad = toks.copy()
+    bad[-1] = dims.vocab_size
+    with pytest.raises(L2Error):
+        m.prefill_chunks(bad, 0, chunk)
+    m.close()
+
+
 @pytest.mark.parametrize("dims,B", [(TINY_GQA, 5), (MID, 33), (MID, 128), (TINY, 37), (GQA8_G64, 5), (GQA8_G64, 64),
                                     (GQA8_G64, 130)],
                          ids=["gqa_g128_b5", "g32_b33", "g32_b128", "mha_g64_b37", "gqa8_g64_b5", "gqa8_g64_b64",
