@@ -608,6 +608,10 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     return L2_OK;
 }
 
+// Rows in flight per stream (P) were measured per shape on whole decode steps.  Where the rows of a block are
+// few (4096 and 11008 inputs: 4 to 8 rows per stream), fewer loads primed in front of x let x arrive sooner,
+// and every instruction of the kernel waits for x: two rows at 4096 inputs (7B +1.2 %), three at 11008 (+0.9 %)
+// and at 13824 through the per-wave form (13B +0.7 %); priming all rows of the block is 15-20 % slower.
 template <int G, int MODE>
 int launch_sg(Q4Launch &L, hipStream_t stream) {
     const int nwk = (L.in / 32 + 63) / 64;
@@ -616,18 +620,18 @@ int launch_sg(Q4Launch &L, hipStream_t stream) {
             case 3:
                 if (plan_cost(L, 3, 5, 4, false) < plan_cost(L, 3, 4, 4, false)) return launch_s<G, 3, 5, false, MODE>(L, stream);
                 return launch_s<G, 3, 4, false, MODE>(L, stream);
-            case 7: return launch_s<G, 7, 2, false, MODE, 5>(L, stream);
+            case 7: return launch_s<G, 7, 2, false, MODE, 3>(L, stream);
             case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, MODE>(L, stream);
         }
     } else if (!L.pair) {
         switch (nwk) {
             case 1: return launch_s<G, 1, 4, false, MODE>(L, stream);
-            case 2: return launch_s<G, 2, 4, false, MODE>(L, stream);
+            case 2: return launch_s<G, 2, 4, false, MODE, 2>(L, stream);
             case 3: // 5120: 20 rows per block are one tile of 5 streams, 60 or so are four tiles either way
                 if (plan_cost(L, 3, 5, 4, false) < plan_cost(L, 3, 4, 4, false)) return launch_s<G, 3, 5, false, MODE>(L, stream);
                 return launch_s<G, 3, 4, false, MODE>(L, stream);
             case 4: return launch_s<G, 4, 4, false, MODE, 2>(L, stream); // 8192: rows of 4 KB; two in flight per stream measured faster than four (q|k|v 13.4 -> 12.2 us, wo 12.1 -> 10.9)
-            case 5: case 6: return launch_s<G, 6, 2, false, MODE>(L, stream);
+            case 5: case 6: return launch_s<G, 6, 2, false, MODE, 3>(L, stream);
             case 7: return launch_s<G, 7, 2, false, MODE, 5>(L, stream); // 13824 -> 5120: 20 rows per block in two tiles
             case 8: return launch_s<G, 8, 2, false, MODE>(L, stream);
             case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, MODE>(L, stream);
