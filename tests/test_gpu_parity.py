@@ -208,6 +208,54 @@ def test_decode_attention_long_context(ops, oracle, n_heads, n_kv, ctx):
     o.close()
 
 
+_VALU_ATTN_SNIPPET = r"""
+import sys, numpy as np
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[2])
+from llama2_rs import ops, checkpoint as ck
+from oracle import oracle_lib as oracle
+worst = 0.0
+for n_heads, n_kv, ctx in ((8, 2, 257), (8, 1, 1000), (8, 1, 70)):
+    dims = ck.Dims(dim=128 * n_heads, hidden_dim=512, n_layers=2, n_heads=n_heads, n_kv_heads=n_kv,
+                   vocab_size=300, seq_len=ctx + 8, group_size=128)
+    img = ck.synth_weights_image(dims, seed=7)
+    m = ops.Model(img, dims)
+    o = oracle.Model(img, dims)
+    o.new_state()
+    m.fill_kv_synthetic(0, ctx, seed=3)
+    ko, vo = o.kv_cache()
+    for l in range(dims.n_layers):
+        k, v = m.read_kv(l, 0, ctx)
+        ko[l, :ctx] = k
+        vo[l, :ctx] = v
+    tok = 11
+    for pos in range(ctx, ctx + 3):
+        want = np.asarray(o.transformer([tok], [pos]), np.float64)
+        got = np.asarray(m.forward([tok], [pos]), np.float64)
+        scale = np.maximum(np.abs(want), np.sqrt(np.mean(want ** 2)) + 1e-30)
+        worst = max(worst, float(np.max(np.abs(got - want) / scale)))
+        tok = oracle.argmax(want)
+        assert int(np.argmax(got)) == tok
+    m.close()
+    o.close()
+print("WORST", worst)
+"""
+
+
+def test_valu_decode_attention_for_grouped_queries():
+    """L2_ATTN_IMPL=valu keeps the vector-ALU decode attention for 4 and 8 query heads per kv head (the matrix-core
+    kernel is the default there): the long-context cases again, in a process of its own."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, L2_ATTN_IMPL="valu")
+    r = subprocess.run([sys.executable, "-c", _VALU_ATTN_SNIPPET, os.path.join(root, "llama2.rs_amd"), root],
+                       capture_output=True, text=True, env=env, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    worst = float(r.stdout.strip().split("WORST")[-1])
+    assert worst < REL_FP32, worst
+
+
 DENSE = ck.Dims(dim=512, hidden_dim=640, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=260,
                 seq_len=80, group_size=0)
 DENSE_WIDE = ck.Dims(dim=256, hidden_dim=9216, n_layers=1, n_heads=2, n_kv_heads=2, vocab_size=64,
