@@ -13,7 +13,8 @@ KV cache are resident in HBM before the timed region starts.
 
 The top level of the JSON line is that run (K and W as given).  Beside it, in
 the same process and the same line, "configs" carries the stated workloads at
-their stated lengths: the 7B decode of 256 tokens after a 16-token prompt, the
+their stated lengths: the standalone 4096x4096 group-128 matvec over 64 weight
+instances, the 7B decode of 256 tokens after a 16-token prompt, the
 7B prefill of a 512-token prompt in chunks of 128 through the MFMA path, the
 13B decode (32 + 256), and the 70B group-64 decode of 128 tokens behind 4096
 cached positions, each with its own roofline object (--configs none skips
@@ -75,6 +76,20 @@ def measured_traffic(model: str, kernels: dict):
     path = os.path.join(ROOT, "profiles", f"q4_matvec_{model}_decode_hbm_counters.txt")
     if not os.path.exists(path):
         return None, f"no counter summary profiles/{os.path.basename(path)}"
+    table = counter_table(path)
+    total = 0
+    for cls in Q4_CLASSES:
+        name = kernels.get(cls, "?") + "(Q4Launch)"
+        for section in ("FETCH_SIZE", "WRITE_SIZE"):
+            if name not in table[section]:
+                return None, (f"profiles/{os.path.basename(path)} holds no {section} reading for {name} ({cls}): "
+                              "it was taken with other kernels, take it again")
+            total += table[section][name]
+    return round(total / len(Q4_CLASSES)), f"profiles/{os.path.basename(path)}"
+
+
+def counter_table(path: str) -> dict:
+    """{"FETCH_SIZE": {kernel: bytes}, "WRITE_SIZE": {...}} of a committed counter summary."""
     table = {"FETCH_SIZE": {}, "WRITE_SIZE": {}}
     section = None
     for line in open(path):
@@ -85,15 +100,83 @@ def measured_traffic(model: str, kernels: dict):
         m = re.match(r"^\s+(\d+)\s+([\d.]+)\s+(\d+)\s+(\S.*)$", line)
         if m and section:
             table[section][m.group(4).strip()] = int(m.group(3))
-    total = 0
-    for cls in Q4_CLASSES:
-        name = kernels.get(cls, "?") + "(Q4Launch)"
-        for section in ("FETCH_SIZE", "WRITE_SIZE"):
-            if name not in table[section]:
-                return None, (f"profiles/{os.path.basename(path)} holds no {section} reading for {name} ({cls}): "
-                              "it was taken with other kernels, take it again")
-            total += table[section][name]
-    return round(total / len(Q4_CLASSES)), f"profiles/{os.path.basename(path)}"
+    return table
+
+
+def matvec_run(np, ops, n_inst: int, iters: int, reps: int, cpu: bool) -> dict:
+    """BASELINE config 0: the standalone GPTQ 4-bit matvec at the 7B q_proj shape (in = out = 4096, group 128,
+    act-order, batch 1), launched back to back over n_inst distinct weight instances (more bytes than the 256 MB
+    memory-side cache holds, so every launch streams its weights from HBM).  Instance 0 is config 0 itself (numpy
+    default_rng(0): AutoGPTQ-layout tensors through the exporter's transform, x ~ N(0,1)) and is checked against
+    the CPU restatement; the others draw the same distributions in the `.bin` layout directly."""
+    from llama2_rs import checkpoint as ck
+    n_in = n_out = 4096
+    G = 128
+    groups = n_in // G
+    rng0 = np.random.default_rng(0)
+    qw0, qz0, sc0, gi0 = ck.synth_qlinear(rng0, n_in, n_out, G, act_order=True)
+    x0 = rng0.standard_normal(n_in).astype(np.float32)
+    qs = [ops.QLinear(qw0, qz0, sc0, gi0, G)]
+    host = [(qw0, qz0, sc0, gi0)]
+    for i in range(1, n_inst):
+        rng = np.random.default_rng(i)
+        qw = rng.integers(0, 1 << 32, size=(n_out, n_in // 8), dtype=np.uint64).astype(np.uint32).view(np.int32)
+        qz = rng.integers(0, 1 << 32, size=(n_out // 8, groups), dtype=np.uint64).astype(np.uint32).view(np.int32)
+        sc = rng.uniform(0.002, 0.02, size=(n_out, groups)).astype(np.float32)
+        gi = np.argsort(rng.permutation(np.arange(n_in) // G), kind="stable").astype(np.int32)
+        qs.append(ops.QLinear(qw, qz, sc, gi, G))
+        if i < 8:
+            host.append((qw, qz, sc, gi))
+    nbytes = q4_bytes(n_in, n_out, G)
+    y_gpu = qs[0].matvec(x0)
+    cadence = sorted(ops.qlinear_bench(qs, iters) / iters * 1e3 for _ in range(reps))  # us per launch, events around the loop
+    us_cad = cadence[len(cadence) // 2]
+    n_disp = min(iters, 1024)
+    us_disp = ops.qlinear_bench_dispatch(qs, n_disp) / n_disp * 1e3               # us per dispatch, its own events
+    kernel = ops.qlinear_kernel(qs[0])
+    traffic, note = None, "no counter summary profiles/q4_matvec_cfg0_hbm_counters.txt"
+    path = os.path.join(ROOT, "profiles", "q4_matvec_cfg0_hbm_counters.txt")
+    if os.path.exists(path):
+        t = counter_table(path)
+        name = kernel + "(Q4Launch)"
+        if name in t["FETCH_SIZE"] and name in t["WRITE_SIZE"]:
+            traffic, note = t["FETCH_SIZE"][name] + t["WRITE_SIZE"][name], "profiles/q4_matvec_cfg0_hbm_counters.txt"
+        else:
+            note = f"profiles/q4_matvec_cfg0_hbm_counters.txt holds no reading for {name}: take it again"
+    gbs = nbytes / us_disp / 1e3
+    out = {
+        "workload": (f"standalone GPTQ 4-bit act-order matvec, in {n_in}, out {n_out}, group {G}, batch 1; {n_inst} distinct "
+                     f"weight instances ({n_inst * nbytes / 1e6:.0f} MB) launched round-robin, {iters} launches x {reps} runs"),
+        "value": round(gbs, 1), "unit": "GB/s", "steps": iters, "warmup": n_inst,
+        "ms_per_step": round(us_disp * 1e-3, 6),
+        "us_per_launch_back_to_back": round(us_cad, 3),
+        "GBs_back_to_back": round(nbytes / us_cad / 1e3, 1),
+        "dtype": "f32",
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": note,
+                     "algorithmic_bytes_per_launch": nbytes, "kernel": kernel,
+                     "duration": "mean of the dispatches' own start/stop events; back-to-back cadence beside it"},
+    }
+    if cpu:
+        from oracle import oracle_lib
+        cores = oracle_lib.num_threads()
+        y_cpu = oracle_lib.qmatvec(qw0, qz0, sc0, gi0, G, x0)
+        scale = np.maximum(np.abs(y_cpu), np.sqrt(np.mean(y_cpu.astype(np.float64) ** 2)))
+        out["max_rel_err_vs_cpu"] = float(np.max(np.abs(y_gpu - y_cpu) / scale))
+        xs = np.random.default_rng(99).standard_normal(n_in).astype(np.float32)
+        n_cpu, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 5.0:
+            for h in host:
+                oracle_lib.qmatvec(*h, G, xs)
+            n_cpu += len(host)
+        t_cpu = (time.perf_counter() - t0) / n_cpu
+        out["cpu_baseline"] = {"value": round(nbytes / t_cpu / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                               "us_per_matvec": round(t_cpu * 1e6, 1),
+                               "sample": f"C restatement of QLinear::matvec<1> (OpenMP over rows, 8-lane AVX2) on {len(host)} of "
+                                         f"the instances round-robin, {n_cpu} matvecs in about 5 s"}
+    for q in qs:
+        q.close()
+    return out
 
 
 class Loaded:
@@ -287,12 +370,15 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="decoded tokens of the CPU sample (0 = sized to ~15 s)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
-                    help="prefill: BASELINE config 2 alone (prompt in chunks through the dequant->fp16 MFMA GEMM, then decode)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "matvec"],
+                    help="prefill: BASELINE config 2 alone (prompt in chunks through the dequant->fp16 MFMA GEMM, then decode); "
+                         "matvec: BASELINE config 0 alone (the standalone 4096x4096 group-128 matvec)")
+    ap.add_argument("--instances", type=int, default=64, help="matvec: distinct weight instances cycled through")
+    ap.add_argument("--iters", type=int, default=2048, help="matvec: launches per timed run")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--chunk", type=int, default=128)
     ap.add_argument("--configs", default=None,
-                    help="which of the stated workloads to run beside the headline: comma list of 1,2,3,4, or none "
+                    help="which of the stated workloads to run beside the headline: comma list of 0,1,2,3,4, or none "
                          "(default: all for the plain 7B run, none otherwise)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -307,11 +393,21 @@ def main() -> int:
         return 2
     plain = a.model == "7B" and not a.layers and not a.group and not a.kv_prefill and a.workload == "decode"
     if a.configs is None:
-        a.configs = "1,2,3,4" if plain else "none"
+        a.configs = "0,1,2,3,4" if plain else "none"
     want = set() if a.configs == "none" else {int(c) for c in a.configs.split(",") if c}
 
     import numpy as np
     from llama2_rs import ops
+
+    if a.workload == "matvec":
+        r = matvec_run(np, ops, a.instances, a.iters, 5, not a.no_cpu_baseline)
+        result = {"metric": "GPTQ matvec HBM GB/s (% of peak) on 1 MI355X", "value": r["value"], "unit": "GB/s", "n_gpus": 1,
+                  "steps": r["steps"], "warmup": r["warmup"], "ms_per_step": r["ms_per_step"], "higher_is_better": True,
+                  "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                  "config": {"workload": r["workload"], "seed": 0}}
+        result.update({k: v for k, v in r.items() if k not in result and k != "workload"})
+        print(json.dumps(result))
+        return 0
 
     M = Loaded(ops, a.model, a.group, a.layers, a.kv_prefill + max(W + K, 16 + 256) + 16, a.seed)
 
@@ -347,6 +443,8 @@ def main() -> int:
     configs = {}
     if want:
         t_all = time.time()
+        if 0 in want:   # config 0: the standalone matvec the GB/s half of the metric is quoted on
+            configs["cfg0_q4_matvec_4096x4096_g128"] = matvec_run(np, ops, 64, 2048, 5, not a.no_cpu_baseline)
         if 1 in want:   # config 1 at its stated length
             configs["cfg1_7B_decode_16+256"] = decode_run(np, M, 16, 256, 0, False, 0)
         if 2 in want:   # config 2: 512-token prompt in chunks of 128 through the MFMA path, then 64 greedy steps

@@ -90,14 +90,6 @@ int l2_preset(const char *model_size, int group_size, l2_dims *out);
  * src/lib.rs:97 asserts the mapped file (after its 28-byte header) to have. */
 size_t l2_weights_bytes(const l2_dims *dims);
 
-/* Fill `buf` (l2_weights_bytes(dims) bytes of host memory) with a random-init
- * weights image in the `.bin` layout: uniform nibbles, scales U[0.002,0.02],
- * act-order g_index (stable argsort of a shuffled i/group_size), norm weights,
- * embedding and classifier N(0, 0.02), rms_eps 1e-5.  Deterministic in `seed`.
- * No counterpart in the reference (it only loads exported checkpoints,
- * export.py:25-122); stands in for one where no checkpoint can be fetched. */
-int l2_synth_image(const l2_dims *dims, uint64_t seed, void *buf, size_t nbytes);
-
 /* LlamaModel::from_file (src/lib.rs:88-104, gpu variant :45-63): open, read
  * the header, check it against `expect` as Config::check_static does
  * (src/constants.rs:94-100: dim, hidden_dim, n_layers, n_heads, vocab_size),
@@ -145,11 +137,6 @@ int l2_state_read_kv(l2_state *s, int layer, int pos0, int npos, float *k_host, 
  * a RunState (the reference clones the boxed struct, src/models.rs:29-42), so
  * that a shared prompt prefix is computed once. */
 int l2_state_write_kv(l2_state *s, int layer, int pos0, int npos, const float *k_host, const float *v_host);
-/* Overwrite cache rows [pos0, pos0+npos) of every layer with a deterministic
- * pattern in (-1, 1) derived from seed: stands in for a long prompt when a
- * benchmark needs a deep cache without paying for its prefill. */
-int l2_state_fill_synthetic(l2_state *s, int pos0, int npos, uint64_t seed);
-
 /* QLinear::convert + QLinearCuda (src/gptq_cuda.rs:70-110): upload the four
  * arrays of one QLinear in `.bin` layout (src/gptq.rs:68-84):
  *   qweight i32[out][in/8], qzeros i32[out/8][groups], scales f32[out][groups],
@@ -246,39 +233,6 @@ int l2_random_sample(l2_random *r, const float *probabilities, int n); /* Random
 int l2_generate(l2_model *m, l2_state *s, const l2_tokenizer *t, const char *prompt, int steps,
                 l2_random *rng, float temperature, int print_tokens, char *out, size_t out_cap,
                 int *n_tokens, int64_t *ms);
-
-/* ---- measurement hooks (no counterpart in the reference: it has no
- * benchmark harness beyond the tok/s line of src/main.rs:62-65) ------------ */
-
-/* Launch the B=1 matvec of qs[0..n) round-robin `iters` times on device-resident
- * random x (no host copies inside the timed region), timed with HIP events on
- * the launch stream.  *ms_total is the elapsed time of all iters launches. */
-int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_total);
-
-/* Decode `n_tokens` greedy steps from (token,pos), the argmax fed back on the
- * device, with HIP events around the whole run on the launch stream; out_ids
- * may be NULL. */
-int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
-                    int32_t *out_ids, float *ms_total);
-
-/* The same loop with a pair of HIP events around every kernel launch (so it
- * runs slower than l2_decode_bench): per kernel class, the summed event time
- * in ms and the number of launches.  Arrays hold l2_kernel_class_count()
- * entries, named by l2_kernel_class_name(). */
-int l2_kernel_class_count(void);
-const char *l2_kernel_class_name(int cls);
-int l2_decode_profile(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
-                      float *ms_by_class, int32_t *launches_by_class);
-
-/* Which kernel each q4 launch class of the decode step runs for this model, as
- * "q4_qkv=<kernel>;q4_wo=<kernel>;q4_w13=<kernel>;q4_w2=<kernel>;" with the names a profiler prints
- * (template arguments included), so that counter readings taken per kernel name can be matched to the
- * launches of a run.  Launches nothing. */
-int l2_model_q4_kernels(l2_model *m, char *out, size_t cap);
-
-/* Plain device-to-device copy of nbytes, iters times: the box's achievable
- * copy bandwidth (bytes moved = 2*nbytes per iteration). */
-int l2_copy_bench(size_t nbytes, int iters, float *ms_total);
 
 #ifdef __cplusplus
 }

@@ -1764,6 +1764,64 @@ extern "C" int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_tot
     return L2_OK;
 }
 
+extern "C" int l2_qlinear_bench_dispatch(l2_qlinear **qs, int n, int iters, float *ms_sum) {
+    if (!qs || n < 1 || iters < 1 || iters > 65536 || !ms_sum) return l2_fail(L2_ERR_ARG, "bad argument");
+    hipStream_t st = qs[0]->stream;
+    for (int i = 0; i < n; i++) {
+        if (!qs[i]) return l2_fail(L2_ERR_ARG, "null qlinear %d", i);
+        L2_TRY(qlinear_scratch(qs[i], 1));
+        L2_TRY(fill_pattern_launch(qs[i]->xg, (size_t)qs[i]->q.in, 17 + i, st));
+    }
+    for (int i = 0; i < n; i++) L2_TRY(q4_one(qs[i]->q, qs[i]->xg, qs[i]->y, 1, st)); // warm-up
+    L2_HIP(hipStreamSynchronize(st));
+    std::vector<hipEvent_t> ev((size_t)iters * 2, nullptr);
+    int rc = L2_OK;
+    for (auto &e : ev)
+        if (rc == L2_OK && hipEventCreate(&e) != hipSuccess) rc = l2_fail(L2_ERR_HIP, "hipEventCreate failed");
+    int launched = 0;
+    for (int it = 0; it < iters && rc == L2_OK; it++) {
+        l2_qlinear *q = qs[it % n];
+        g_q4_prof.start = ev[2 * (size_t)it];
+        g_q4_prof.stop = ev[2 * (size_t)it + 1];
+        g_q4_prof.armed = true;
+        rc = q4_one(q->q, q->xg, q->y, 1, st);
+        if (rc == L2_OK && g_q4_prof.armed) rc = l2_fail(L2_ERR_ARG, "this form of the kernel takes no dispatch events");
+        g_q4_prof.armed = false;
+        if (rc == L2_OK) launched++;
+    }
+    const hipError_t es = hipStreamSynchronize(st);
+    double sum = 0.0;
+    for (int it = 0; it < launched && rc == L2_OK && es == hipSuccess; it++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, ev[2 * (size_t)it], ev[2 * (size_t)it + 1]) != hipSuccess)
+            rc = l2_fail(L2_ERR_HIP, "hipEventElapsedTime failed on dispatch %d", it);
+        sum += ms;
+    }
+    for (auto &e : ev)
+        if (e) (void)hipEventDestroy(e);
+    if (rc != L2_OK) return rc;
+    if (es != hipSuccess) return l2_fail(L2_ERR_HIP, "matvec bench: %s", hipGetErrorString(es));
+    *ms_sum = (float)sum;
+    return L2_OK;
+}
+
+extern "C" int l2_qlinear_kernel(l2_qlinear *q, char *out, size_t cap) {
+    if (!q || !out || cap < 2) return l2_fail(L2_ERR_ARG, "bad argument");
+    out[0] = '\0';
+    const float *some = (const float *)q->bufs[2]; // only null / non-null matters for the choice of kernel
+    Q4Launch L = launch_of(q->q, 1, 0.f);
+    L.m[0] = mat_of(q->q, some, nullptr, nullptr);
+    g_q4_name.buf = out;
+    g_q4_name.cap = (int)cap;
+    g_q4_name.armed = true;
+    const int rc = q4_matvec_launch(L, q->stream);
+    const bool answered = !g_q4_name.armed;
+    g_q4_name.armed = false;
+    L2_TRY(rc);
+    if (!answered) return l2_fail(L2_ERR_ARG, "the launcher did not name its kernel");
+    return L2_OK;
+}
+
 extern "C" int l2_decode_bench(l2_model *m, l2_state *s, int32_t token, int32_t pos, int n_tokens,
                                int32_t *out_ids, float *ms_total) {
     if (!m || !s || !ms_total || n_tokens < 1) return l2_fail(L2_ERR_ARG, "bad argument");

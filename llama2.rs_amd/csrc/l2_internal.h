@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../../include/llama2_hip.h"
+#include "../../include/llama2_hip_bench.h"
 
 // Compute units of the current device (256 on MI355X); asked once.
 inline int cu_count() {

@@ -86,6 +86,8 @@ SIGNATURES = {
     "l2_generate": (_I, [_VP, _VP, _VP, C.c_char_p, _I, _VP, C.c_float, _I, _VP, _SZ, C.POINTER(_I),
                          C.POINTER(C.c_int64)]),
     "l2_qlinear_bench": (_I, [C.POINTER(_VP), _I, _I, C.POINTER(C.c_float)]),
+    "l2_qlinear_bench_dispatch": (_I, [C.POINTER(_VP), _I, _I, C.POINTER(C.c_float)]),
+    "l2_qlinear_kernel": (_I, [_VP, C.c_char_p, _SZ]),
     "l2_decode_bench": (_I, [_VP, _VP, C.c_int32, C.c_int32, _I, _VP, C.POINTER(C.c_float)]),
     "l2_kernel_class_count": (_I, []),
     "l2_kernel_class_name": (C.c_char_p, [_I]),

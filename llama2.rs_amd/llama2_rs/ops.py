@@ -113,6 +113,21 @@ def qlinear_bench(qs, iters: int) -> float:
     return ms.value
 
 
+def qlinear_bench_dispatch(qs, iters: int) -> float:
+    """Sum in milliseconds of the `iters` dispatch durations (each launch's own start/stop events)."""
+    arr = (C.c_void_p * len(qs))(*[q.h for q in qs])
+    ms = C.c_float()
+    check(lib().l2_qlinear_bench_dispatch(arr, len(qs), iters, C.byref(ms)))
+    return ms.value
+
+
+def qlinear_kernel(q) -> str:
+    """Name (as a profiler prints it) of the kernel a B=1 matvec of q runs."""
+    buf = C.create_string_buffer(256)
+    check(lib().l2_qlinear_kernel(q.h, buf, 256))
+    return buf.value.decode()
+
+
 def copy_bench(nbytes: int, iters: int) -> float:
     ms = C.c_float()
     check(lib().l2_copy_bench(nbytes, iters, C.byref(ms)))

@@ -24,6 +24,12 @@
  *                  reference and its Rust cannot be built here: parity with
  *                  the reference's in-place update order is by reading only.
  *   or_argmax      duplicates resolve to the last index.
+ *   or_str_lookup, or_bpe_encode  the reference's test (tests/test_tokenizer.py:8-23)
+ *                  asserts equality with the SentencePiece BPE encoding of the same
+ *                  vocabulary; tests/test_oracle_tokenizer.py builds that SentencePiece
+ *                  model from tokenizer.bin (pieces and scores as they stand) and compares
+ *                  ids on the reference's two prompts and on seeded ordinary text; a toy
+ *                  vocabulary checks the merge order by hand and the ids-from-260-first rule.
  *   or_transformer, or_generate_greedy  parity unpinned by any reference
  *                  fixture (the reference holds no checkpoint and no expected
  *                  tokens); pinned structurally: batched prefill == token by
@@ -567,4 +573,65 @@ int or_generate_greedy(const or_model *m, or_state *state, const int *prompt, in
     free(logits);
     or_state_free(own);
     return n;
+}
+
+/* ---- tokenizer --------------------------------------------------------------
+ * The vocabulary as Tokenizer::load leaves it (src/tokenizer.rs:22-37): n strings,
+ * string i = bytes[off[i] .. off[i+1]), and their scores. */
+
+/* util::str_lookup (src/util.rs:29-37): the first perfect match among ids 260.., and only if there is none
+ * the first match from the start.  A linear scan, as in the reference.  -1 = None. */
+int or_str_lookup(const char *str, int len, const char *bytes, const int32_t *off, int n) {
+    for (int i = 260; i < n; i++)
+        if (off[i + 1] - off[i] == len && memcmp(bytes + off[i], str, (size_t)len) == 0) return i;
+    for (int i = 0; i < n; i++)
+        if (off[i + 1] - off[i] == len && memcmp(bytes + off[i], str, (size_t)len) == 0) return i;
+    return -1;
+}
+
+static int utf8_len(unsigned char c) { return c < 0x80 ? 1 : (c >> 5) == 6 ? 2 : (c >> 4) == 14 ? 3 : 4; }
+
+/* Tokenizer::bpe_encode (src/tokenizer.rs:46-108).  text: UTF-8, text_len bytes.  Returns the number of
+ * tokens written to `tokens` (capacity cap >= number of characters), -1 if a character is not in the
+ * vocabulary (the reference's expect("not good")), -2 if cap is too small or the text is empty (the
+ * reference's `0..(tokens.len() - 1)` underflows on an empty vector). */
+int or_bpe_encode(const char *text, int text_len, const char *bytes, const int32_t *off, const float *scores,
+                  int n, int32_t *tokens, int cap) {
+    int nt = 0;
+    /* :52-61 every character (Unicode scalar value) on its own */
+    for (int i = 0; i < text_len;) {
+        int l = utf8_len((unsigned char)text[i]);
+        if (i + l > text_len) l = text_len - i;
+        const int id = or_str_lookup(text + i, l, bytes, off, n);
+        if (id < 0) return -1;
+        if (nt >= cap) return -2;
+        tokens[nt++] = id;
+        i += l;
+    }
+    if (nt == 0) return -2;
+    char *buf = (char *)malloc(1 << 16);
+    if (!buf) return -2;
+    for (;;) { /* :64-107 merge the best consecutive pair until none is in the vocabulary */
+        float best_score = -1e10f;
+        int best_id = 0, best_idx = -1;
+        for (int i = 0; i < nt - 1; i++) {
+            const int a = tokens[i], b = tokens[i + 1];
+            const int la = off[a + 1] - off[a], lb = off[b + 1] - off[b];
+            if (la + lb > (1 << 16)) continue;
+            memcpy(buf, bytes + off[a], (size_t)la);
+            memcpy(buf + la, bytes + off[b], (size_t)lb);
+            const int id = or_str_lookup(buf, la + lb, bytes, off, n);
+            if (id >= 0 && scores[id] > best_score) { /* strict: the leftmost of equal scores stays */
+                best_score = scores[id];
+                best_id = id;
+                best_idx = i;
+            }
+        }
+        if (best_idx < 0) break;
+        tokens[best_idx] = best_id;
+        for (int i = best_idx + 1; i < nt - 1; i++) tokens[i] = tokens[i + 1];
+        nt--;
+    }
+    free(buf);
+    return nt;
 }

@@ -67,6 +67,10 @@ def lib() -> C.CDLL:
         L.or_argmax.restype = C.c_int
         L.or_argmax.argtypes = [C.c_void_p, C.c_int]
         L.or_accum.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        L.or_str_lookup.restype = C.c_int
+        L.or_str_lookup.argtypes = [C.c_char_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int]
+        L.or_bpe_encode.restype = C.c_int
+        L.or_bpe_encode.argtypes = [C.c_char_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
         L.or_num_threads.restype = C.c_int
         L.or_set_num_threads.argtypes = [C.c_int]
         _lib = L
@@ -161,6 +165,56 @@ def attention(queries, value_cache, key_cache, pos, n_heads: int, n_kv_heads: in
 def argmax(v) -> int:
     v = _f32(v)
     return lib().or_argmax(_p(v), v.shape[0])
+
+
+def read_tokenizer_file(path: str, vocab_size: int):
+    """Tokenizer::load (src/tokenizer.rs:22-37): i32 max_token_length, then vocab_size x {f32 score, i32 len,
+    bytes}.  Returns (list of bytes, float32 scores, max_token_length)."""
+    import struct
+    data = open(path, "rb").read()
+    (max_len,) = struct.unpack_from("<i", data, 0)
+    off, vocab, scores = 4, [], np.empty(vocab_size, np.float32)
+    for i in range(vocab_size):
+        sc, ln = struct.unpack_from("<fi", data, off)
+        off += 8
+        vocab.append(data[off:off + ln])
+        off += ln
+        scores[i] = sc
+    return vocab, scores, max_len
+
+
+class Tokenizer:
+    """Tokenizer (src/tokenizer.rs:13-108) over a vocabulary given as a list of byte strings and scores."""
+
+    def __init__(self, vocab, scores):
+        self.vocab = [bytes(v) for v in vocab]
+        self.scores = _f32(scores)
+        assert len(self.vocab) == self.scores.shape[0]
+        self._bytes = np.frombuffer(b"".join(self.vocab) + b"\0", np.uint8).copy()
+        self._off = np.zeros(len(self.vocab) + 1, np.int32)
+        np.cumsum([len(v) for v in self.vocab], out=self._off[1:])
+
+    @classmethod
+    def from_file(cls, path: str, vocab_size: int = 32000):
+        vocab, scores, _ = read_tokenizer_file(path, vocab_size)
+        return cls(vocab, scores)
+
+    def str_lookup(self, s) -> int:
+        """util::str_lookup (src/util.rs:29-37); -1 for None."""
+        b = s.encode("utf-8") if isinstance(s, str) else bytes(s)
+        return lib().or_str_lookup(b, len(b), _p(self._bytes), _p(self._off), len(self.vocab))
+
+    def bpe_encode(self, text) -> list:
+        """Tokenizer::bpe_encode (src/tokenizer.rs:46-108)."""
+        b = text.encode("utf-8") if isinstance(text, str) else bytes(text)
+        out = np.empty(max(len(b), 1), np.int32)
+        n = lib().or_bpe_encode(b, len(b), _p(self._bytes), _p(self._off), _p(self.scores), len(self.vocab),
+                                _p(out), out.shape[0])
+        if n == -1:
+            raise ValueError("a character of the text is not in the vocabulary")
+        if n < 0:
+            raise ValueError("empty text")
+        return out[:n].tolist()
 
 
 class Model:

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "../../include/llama2_hip.h"
+#include "../../include/llama2_hip_bench.h"
 
 #define REQUIRE(cond)                                                     \
     do {                                                                  \

@@ -14,7 +14,7 @@ GOLD = os.path.join(ROOT, "tests", "golden")
 def test_library_exports_every_declared_symbol():
     from llama2_rs import _lib
     L = _lib.lib()
-    header = open(os.path.join(ROOT, "include", "llama2_hip.h")).read()
+    header = "".join(open(os.path.join(ROOT, "include", h)).read() for h in ("llama2_hip.h", "llama2_hip_bench.h"))
     declared = set(re.findall(r"\b(l2_[a-z0-9_]+)\s*\(", header))
     assert declared, "no declarations found"
     for name in sorted(declared):
