@@ -159,7 +159,11 @@ int l2_qlinear_matvec(l2_qlinear *q, const float *x_host, int B, float *y_host);
  * device array of L2_MATVEC_DEVICE_MAX_ELEMS floats (4 MiB) that each GPU holds until the process
  * ends, so B * in must not exceed that count (L2_ERR_RANGE otherwise).  All calls on one GPU share the array:
  * calls that overlap in time on one GPU (two streams, two threads) race; serialise them.  y equals
- * l2_qlinear_matvec's bit for bit. */
+ * l2_qlinear_matvec's bit for bit.  What a first launch does besides enqueueing (loading the code object on the
+ * device, raising the kernel's LDS limit, resolving the array's address) l2_qlinear_create has already done, with
+ * the device that is current at that time: a handle is used on the device it was created on, and every call
+ * here, the first included, may be made while hip_stream is being captured into a graph.  Nothing it enqueues
+ * is a memset node. */
 #define L2_MATVEC_DEVICE_MAX_ELEMS (1u << 20)
 int l2_qlinear_matvec_device(l2_qlinear *q, const float *x_dev, int B, float *y_dev, void *hip_stream);
 

@@ -68,6 +68,13 @@ int l2_decode_profile(l2_model *m, l2_state *s, int32_t token, int32_t pos, int 
  * launches of a run.  Launches nothing. */
 int l2_model_q4_kernels(l2_model *m, char *out, size_t cap);
 
+/* What the B=1 q4 launcher would do for a shape, without a device and without launching: n_mats (1..3) matrices
+ * of `in` inputs and out[i] outputs in one launch (pair != 0: a w1|w3 pair with the SiLU gate behind), with
+ * (norm != 0) or without an rmsnorm in front.  kernel receives the kernel's name as a profiler prints it;
+ * geometry[4] receives {blocks, threads per block, rows per block, dynamic LDS bytes}. */
+int l2_q4_plan(int in, const int32_t *out, int n_mats, int group_size, int pair, int norm, char *kernel, size_t cap,
+               int32_t *geometry);
+
 /* Plain device-to-device copy of nbytes, iters times: the box's achievable
  * copy bandwidth (bytes moved = 2*nbytes per iteration). */
 int l2_copy_bench(size_t nbytes, int iters, float *ms_total);

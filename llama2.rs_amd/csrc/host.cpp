@@ -737,9 +737,16 @@ extern "C" int l2_model_set_prefill_mode(l2_model *m, int mode) {
 
 static int ensure_batch_mfma(l2_model *m, int B);
 
+// Nothing may be running on either of the model's streams when a buffer they use is freed.
+static int drain_streams(l2_model *m) {
+    L2_HIP(hipStreamSynchronize(m->stream));
+    if (m->stream2) L2_HIP(hipStreamSynchronize(m->stream2));
+    return L2_OK;
+}
+
 static int ensure_batch(l2_model *m, int B) {
     if (B <= m->cap_B) return L2_OK;
-    L2_HIP(hipStreamSynchronize(m->stream));
+    L2_TRY(drain_streams(m));
     m->buf_epoch++;
     float **bufs[] = {&m->x, &m->xq, &m->xk, &m->xv, &m->qv, &m->kv, &m->vv, &m->attg, &m->x1, &m->x3, &m->hg};
     for (float **b : bufs) {
@@ -896,6 +903,23 @@ static int check_qlinear_shape(int in, int out, int g) {
     return L2_OK;
 }
 
+static int qlinear_scratch(l2_qlinear *q, int B);
+static int scratch_ptr(float **out);
+
+// Everything a later launch of this layer's operator would otherwise do on first use, done once here and waited
+// for: the code object is loaded on this device, the kernel's dynamic-LDS limit is raised, the fixed scratch
+// array's address is resolved.  A call made under stream capture afterwards only enqueues kernels.
+static int qlinear_warm_up(l2_qlinear *q) {
+    L2_TRY(qlinear_scratch(q, 1));
+    float *fixed = nullptr;
+    L2_TRY(scratch_ptr(&fixed));
+    L2_HIP(hipMemsetAsync(q->x, 0, (size_t)q->q.in * 4, q->stream));
+    L2_TRY(gather_launch(q->xg, q->x, q->q.g_index, q->q.in, 1, q->stream));
+    L2_TRY(q4_one(q->q, q->xg, q->y, 1, q->stream));
+    L2_HIP(hipStreamSynchronize(q->stream));
+    return L2_OK;
+}
+
 extern "C" int l2_qlinear_create(const int32_t *qweight, const int32_t *qzeros, const float *scales,
                                  const int32_t *g_index, int in, int out, int group_size, l2_qlinear **ql) {
     if (!qweight || !qzeros || !scales || !g_index || !ql) return l2_fail(L2_ERR_ARG, "null argument");
@@ -931,6 +955,11 @@ extern "C" int l2_qlinear_create(const int32_t *qweight, const int32_t *qzeros, 
     q->q.out = out;
     q->q.groups = groups;
     q->q.group_size = group_size;
+    const int rc = qlinear_warm_up(q);
+    if (rc != L2_OK) {
+        l2_qlinear_free(q);
+        return rc;
+    }
     *ql = q;
     return L2_OK;
 }
@@ -1273,7 +1302,7 @@ static int forward_enqueue_dense(l2_model *m, l2_state *s, int B, int max_pos, b
 
 static int ensure_batch_mfma(l2_model *m, int B) {
     if (B <= m->cap_B_mfma) return L2_OK;
-    L2_HIP(hipStreamSynchronize(m->stream));
+    L2_TRY(drain_streams(m));
     void **bufs[] = {&m->h16a, &m->h16b, &m->h16c, (void **)&m->hb, (void **)&m->hb2, (void **)&m->ssb,
                      (void **)&m->gemm_ws};
     m->gemm_ws_floats = 0;
@@ -1463,7 +1492,7 @@ static int ensure_prefill_pipeline(l2_model *m, int B, int n) {
         m->cap_pf = n;
     }
     if (B <= m->cap_B_alt) return L2_OK;
-    L2_HIP(hipStreamSynchronize(m->stream2));
+    L2_TRY(drain_streams(m));
     l2_model::ChunkBufs &a = m->alt;
     void **bufs[] = {(void **)&a.x, (void **)&a.xq, (void **)&a.xk, (void **)&a.xv, (void **)&a.qv, (void **)&a.kv,
                      (void **)&a.vv, &a.h16a, &a.h16b, &a.h16c, (void **)&a.hb, (void **)&a.hb2, (void **)&a.ssb,
@@ -1522,30 +1551,47 @@ extern "C" int l2_prefill_chunks(l2_model *m, l2_state *s, const int32_t *tokens
     L2_HIP(hipStreamSynchronize(m->stream));
     L2_HIP(hipMemcpy(m->pf_tok, tokens, (size_t)n * 4, hipMemcpyHostToDevice));
     L2_HIP(hipMemcpy(m->pf_pos, pos.data(), (size_t)n * 4, hipMemcpyHostToDevice));
-    int c = 0;
-    for (int c0 = 0; c0 < n; c0 += chunk, c++) {
-        const int B = std::min(chunk, n - c0);
-        const int max_pos = pos0 + c0 + B - 1;
-        if (mfma && B > 1) {
-            l2_model::ChunkBufs b = (c & 1) ? m->alt : primary_bufs(m);
-            b.dtok = m->pf_tok + c0, b.dpos = m->pf_pos + c0;
-            hipStream_t st = (c & 1) ? m->stream2 : m->stream;
-            L2_TRY(forward_enqueue_mfma(m, s, B, max_pos, b, st, m->pf_ev[c & 1].data(),
-                                        c > 0 ? m->pf_ev[(c - 1) & 1].data() : nullptr));
-        } else {
-            // one token left over, or the fp32 mode: the fp32 kernels on the model's stream, behind everything
-            if (c > 0 && mfma) {
-                L2_HIP(hipEventRecord(m->pf_join, m->stream2));
-                L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+    // Everything that is enqueued on the two streams; a failure half-way returns through the caller below, which
+    // first waits for what earlier chunks already have in flight on either stream.
+    auto enqueue_all = [&]() -> int {
+        int c = 0;
+        for (int c0 = 0; c0 < n; c0 += chunk, c++) {
+            const int B = std::min(chunk, n - c0);
+            const int max_pos = pos0 + c0 + B - 1;
+            if (mfma && B > 1) {
+                l2_model::ChunkBufs b = (c & 1) ? m->alt : primary_bufs(m);
+                b.dtok = m->pf_tok + c0, b.dpos = m->pf_pos + c0;
+                hipStream_t st = (c & 1) ? m->stream2 : m->stream;
+                L2_TRY(forward_enqueue_mfma(m, s, B, max_pos, b, st, m->pf_ev[c & 1].data(),
+                                            c > 0 ? m->pf_ev[(c - 1) & 1].data() : nullptr));
+            } else {
+                // one token left over, or the fp32 mode: the fp32 kernels on the model's stream, behind everything
+                if (c > 0 && mfma) {
+                    L2_HIP(hipEventRecord(m->pf_join, m->stream2));
+                    L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+                }
+                L2_HIP(hipMemcpyAsync(m->dtok, m->pf_tok + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
+                L2_HIP(hipMemcpyAsync(m->dpos, m->pf_pos + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
+                L2_TRY(forward_enqueue(m, s, B, max_pos, false));
             }
-            L2_HIP(hipMemcpyAsync(m->dtok, m->pf_tok + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
-            L2_HIP(hipMemcpyAsync(m->dpos, m->pf_pos + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
-            L2_TRY(forward_enqueue(m, s, B, max_pos, false));
         }
-    }
-    if (mfma) {
-        L2_HIP(hipEventRecord(m->pf_join, m->stream2));
-        L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+        if (mfma) {
+            L2_HIP(hipEventRecord(m->pf_join, m->stream2));
+            L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+        }
+        return L2_OK;
+    };
+    const int rc = enqueue_all();
+    if (rc != L2_OK) {
+        // kernels of earlier chunks may still be writing cache rows and chunk buffers on both streams: nothing
+        // returns to the caller (who may reset the state or free the model next) before they are done.  The
+        // error text of the failure that brought us here is kept.
+        char keep[sizeof g_err];
+        memcpy(keep, g_err, sizeof keep);
+        (void)hipStreamSynchronize(m->stream);
+        if (m->stream2) (void)hipStreamSynchronize(m->stream2);
+        memcpy(g_err, keep, sizeof keep);
+        return rc;
     }
     L2_HIP(hipStreamSynchronize(m->stream));
     return L2_OK;
@@ -1899,6 +1945,46 @@ extern "C" int l2_model_q4_kernels(l2_model *m, char *out, size_t cap) {
     }
     if (all.size() + 1 > cap) return l2_fail(L2_ERR_ARG, "buffer of %zu bytes, %zu needed", cap, all.size() + 1);
     memcpy(out, all.c_str(), all.size() + 1);
+    return L2_OK;
+}
+
+extern "C" int l2_q4_plan(int in, const int32_t *out, int n_mats, int group_size, int pair, int norm, char *kernel,
+                          size_t cap, int32_t *geometry) {
+    if (!out || !kernel || cap < 2 || !geometry || n_mats < 1 || n_mats > 3) return l2_fail(L2_ERR_ARG, "bad argument");
+    if (group_size != 32 && group_size != 64 && group_size != 128) return l2_fail(L2_ERR_ARG, "group size %d", group_size);
+    if (in <= 0 || in % 32 || in % group_size) return l2_fail(L2_ERR_ARG, "in=%d", in);
+    static const float dummy[4] = {0.f, 0.f, 0.f, 0.f}; // only null / non-null matters: nothing is launched
+    Q4Launch L{};
+    L.n_mats = n_mats;
+    L.in = in;
+    L.groups = in / group_size;
+    L.group_size = group_size;
+    L.batch = 1;
+    L.pair = pair ? 1 : 0;
+    L.eps = 1e-5f;
+    L.e.kind = pair ? Q4_EPI_SCATTER_ONLY : Q4_EPI_STORE;
+    for (int i = 0; i < n_mats; i++) {
+        if (out[i] <= 0 || out[i] % 8) return l2_fail(L2_ERR_ARG, "out[%d]=%d", i, out[i]);
+        L.m[i].x = dummy;
+        L.m[i].wn = norm ? dummy : nullptr;
+        L.m[i].out = out[i];
+    }
+    kernel[0] = '\0';
+    g_q4_name = Q4NameHook{};
+    g_q4_name.buf = kernel;
+    g_q4_name.cap = (int)cap;
+    g_q4_name.armed = true;
+    const int rc = q4_matvec_launch(L, nullptr);
+    const bool answered = !g_q4_name.armed;
+    g_q4_name.armed = false;
+    L2_TRY(rc);
+    if (!answered) return l2_fail(L2_ERR_ARG, "the launcher did not name its kernel");
+    geometry[0] = g_q4_name.grid, geometry[1] = g_q4_name.block, geometry[2] = g_q4_name.rows_per_block;
+    geometry[3] = (int32_t)g_q4_name.lds;
+    // every row of every matrix belongs to exactly one block, and the blocks of all matrices fit the grid
+    long blocks = 0;
+    for (int i = 0; i < (pair ? 1 : n_mats); i++) blocks += (out[i] + geometry[2] - 1) / geometry[2];
+    if (blocks != geometry[0]) return l2_fail(L2_ERR_ARG, "plan: %ld row blocks for a grid of %d", blocks, geometry[0]);
     return L2_OK;
 }
 

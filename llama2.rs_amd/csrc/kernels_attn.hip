@@ -64,6 +64,11 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Floats per row of the LDS tiles in which rows of lanes, waves and splits meet: the 128 partial outputs, then
+// (m, l).  The outputs are stored four at a time (16-byte LDS stores), so a row starts on a 16-byte boundary.
+constexpr int kCombRow = 128 + 4;
+static_assert(kCombRow * sizeof(float) % 16 == 0, "rows of the merge tiles are written with 16-byte stores");
+
 // Layout of a block: NWV waves x 4 rows of 16 lanes.  One row of lanes handles
 // one timestep at a time, each lane 8 of the 128 head dimensions; a block
 // covers 4 NWV timesteps per step and PD steps per tile, all of a tile's loads
@@ -83,10 +88,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const AttnDecode 
     // step, 160 at 8 heads, a fifth of the kernel at long contexts.
     constexpr bool kRowsInLds = QG >= 4;
     constexpr int NR = kRowsInLds ? NWV * 4 : NWV; // partial results that meet in LDS
-    __shared__ float comb_s[kRowsInLds ? 1 : NWV][QG][HS + 2];
+    __shared__ __align__(16) float comb_s[kRowsInLds ? 1 : NWV][QG][kCombRow];
     __shared__ float wts[QG][16], m_all[QG], den_all[QG];
-    extern __shared__ float comb_d[]; // [NR][QG][HS + 2] when kRowsInLds
-    float(*comb)[QG][HS + 2] = kRowsInLds ? reinterpret_cast<float(*)[QG][HS + 2]>(comb_d) : comb_s;
+    extern __shared__ __align__(16) float comb_d[]; // [NR][QG][kCombRow] when kRowsInLds
+    float(*comb)[QG][kCombRow] = kRowsInLds ? reinterpret_cast<float(*)[QG][kCombRow]>(comb_d) : comb_s;
     pin_args(A);
     const int kvh = blockIdx.x, sp = blockIdx.y;
     const int pos = A.dpos ? A.dpos[0] : A.pos;
@@ -405,7 +410,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(const AttnDeco
     static_assert(QG == 4 || QG == 8, "the query heads of a kv head fill part of the 16 columns of a tile");
     __shared__ float qs[QG * HS];
     __shared__ float kvnew[2][HS];
-    __shared__ float comb[NWV][QG][HS + 2];
+    __shared__ __align__(16) float comb[NWV][QG][kCombRow];
     pin_args(A);
     const int kvh = blockIdx.x, sp = blockIdx.y;
     const int pos = A.dpos ? A.dpos[0] : A.pos;
@@ -661,7 +666,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(float *__restrict__ o
                                                             int n_kv_heads, int B) {
     constexpr int HS = 128, NQ = 8, QPB = NQ / QG, PD = 2, TSTEP = 16;
     __shared__ float qs[NQ * HS];
-    __shared__ float comb[4][NQ][HS + 2];
+    __shared__ __align__(16) float comb[4][NQ][kCombRow];
     __shared__ int pj_s[NQ];
     const int kvh = blockIdx.x, qb = blockIdx.y;
     const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
@@ -1096,14 +1101,10 @@ int attn_launch_qg(const AttnDecode &a, hipStream_t st) {
             return L2_OK;
         }
     }
-    constexpr size_t lds = QG >= 4 ? (size_t)16 * QG * 130 * sizeof(float) : 0; // the partial results of 16 rows
+    constexpr size_t lds = QG >= 4 ? (size_t)16 * QG * kCombRow * sizeof(float) : 0; // the partial results of 16 rows
     if (lds > 48 * 1024) {
-        static bool raised = false; // per instantiation
-        if (!raised) {
-            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_decode_kernel<QG, 4>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            raised = true;
-        }
+        static LdsLimit limit; // per instantiation
+        L2_TRY(limit.ensure(reinterpret_cast<const void *>(attn_decode_kernel<QG, 4>), lds));
     }
     hipLaunchKernelGGL((attn_decode_kernel<QG, 4>), dim3(a.n_kv_heads, a.n_splits), dim3(256), lds, st, a);
     L2_HIP(hipGetLastError());
@@ -1141,13 +1142,8 @@ int attention_launch(float *out, void *out_f16, const float *q, const float *kca
         constexpr size_t lds = (size_t)(128 * 33 + 8 * 32 * 132) * sizeof(float);
         dim3 grid(n_kv_heads, (B * qg + 31) / 32), block(512);
         auto launch = [&](auto kern) {
-            static bool raised = false; // per instantiation
-            if (!raised) {
-                if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        (int)lds) != hipSuccess)
-                    return l2_fail(L2_ERR_HIP, "attention: %zu bytes of LDS refused", lds);
-                raised = true;
-            }
+            static LdsLimit limit; // per instantiation (the lambda is generic: one body per kernel)
+            L2_TRY(limit.ensure(reinterpret_cast<const void *>(kern), lds));
             hipLaunchKernelGGL(kern, grid, block, lds, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads,
                                n_kv_heads, B, max_pos);
             return (int)L2_OK;

@@ -334,13 +334,10 @@ int dense_launch(const DenseArgs &a0, hipStream_t st) {
     if (blocks > need) blocks = need;
     const size_t lds = (size_t)a.n_pass * KI * 64 * 16;
     dim3 grid(blocks, a.batch), block(256);
-    if (lds > 48 * 1024) {
-        static size_t raised = 0;
-        if (lds > raised) {
-            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(dense_matvec_kernel<32>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            raised = lds;
-        }
+    if (lds > 48 * 1024) { // only rows of more than one pass, which run with KI = 32
+        if (KI != 32) return l2_fail(L2_ERR_ARG, "dense matvec: in=%d out=%d needs %zu B of LDS with %d loads per pass", a.in, a.out, lds, KI);
+        static LdsLimit limit;
+        L2_TRY(limit.ensure(reinterpret_cast<const void *>(dense_matvec_kernel<32>), lds));
     }
     switch (KI) {
         case 4: hipLaunchKernelGGL(dense_matvec_kernel<4>, grid, block, lds, st, a); break;

@@ -224,16 +224,13 @@ int launch_t(Q4Launch &L, hipStream_t stream) {
     if (g_q4_name.armed) {
         g_q4_name.armed = false;
         snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_matvec_kernel<%d, %d, %d, %s>", G, R, NW, PAIR ? "true" : "false");
+        g_q4_name.grid = total, g_q4_name.block = NW * 64, g_q4_name.rows_per_block = NW * R, g_q4_name.lds = lds;
         return L2_OK;
     }
     if (lds + 256 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
-    if (lds > 64 * 1024) {
-        static size_t raised = 0; // per instantiation: the largest dynamic LDS size allowed so far
-        if (lds > raised) {
-            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            raised = lds;
-        }
+    if (lds > 48 * 1024) {
+        static LdsLimit limit; // per instantiation
+        L2_TRY(limit.ensure(reinterpret_cast<const void *>(kern), lds));
     }
     dim3 grid(total, L.batch), block(NW * 64);
     if (g_q4_prof.armed) {

@@ -735,12 +735,8 @@ int silu_scatter_launch(float *out, void *out_f16, const float *a, const float *
     if (out_f16) {
         if (!scatter || n % 8 || (size_t)n * 2 > 60 * 1024)
             return l2_fail(L2_ERR_ARG, "silu gate (fp16): n=%d needs a permutation and at most 60 KB of LDS", n);
-        static size_t raised = 48 * 1024;
-        if ((size_t)n * 2 > raised) {
-            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(silu_scatter_f16_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, n * 2));
-            raised = (size_t)n * 2;
-        }
+        static LdsLimit limit(48 * 1024);
+        L2_TRY(limit.ensure(reinterpret_cast<const void *>(silu_scatter_f16_kernel), (size_t)n * 2));
         hipLaunchKernelGGL(silu_scatter_f16_kernel, dim3(B), dim3(1024), (size_t)n * 2, st, (_Float16 *)out_f16, a, c, scatter, n);
     } else {
         hipLaunchKernelGGL(silu_scatter_kernel, dim3((n + 255) / 256, B), dim3(256), 0, st, out, a, c, scatter, n);
@@ -755,12 +751,8 @@ int gemm_residual_norm_prep_launch(const ResNormPrep &A, hipStream_t st) {
     if (A.n == 0) return l2_fail(L2_ERR_ARG, "residual epilogue: no consumer");
     const size_t lds = (size_t)A.n * A.out * sizeof(_Float16);
     if (A.out % 8 || lds > 60 * 1024) return l2_fail(L2_ERR_ARG, "residual epilogue: %d outputs x %d consumers", A.out, A.n);
-    static size_t raised = 48 * 1024;
-    if (lds > raised) {
-        L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_residual_norm_prep_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        raised = lds;
-    }
+    static LdsLimit limit(48 * 1024);
+    L2_TRY(limit.ensure(reinterpret_cast<const void *>(gemm_residual_norm_prep_kernel), lds));
     hipLaunchKernelGGL(gemm_residual_norm_prep_kernel, dim3(A.B), dim3(1024), lds, st, A);
     L2_HIP(hipGetLastError());
     return L2_OK;

@@ -587,15 +587,12 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
         g_q4_name.armed = false;
         snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_stream_kernel<%d, %d, %d, %s, %d, %d>", G, NWK, S,
                  PAIR ? "true" : "false", MODE, P);
+        g_q4_name.grid = total, g_q4_name.block = NW * 64, g_q4_name.rows_per_block = rpb, g_q4_name.lds = lds;
         return L2_OK;
     }
     if (lds > 48 * 1024) {
-        static size_t raised = 0; // per instantiation
-        if (lds > raised) {
-            L2_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            raised = lds;
-        }
+        static LdsLimit limit; // per instantiation
+        L2_TRY(limit.ensure(reinterpret_cast<const void *>(kern), lds));
     }
     dim3 grid(total, L.batch), block(NW * 64);
     if (g_q4_prof.armed) {

@@ -7,7 +7,10 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <mutex>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "../../include/llama2_hip.h"
@@ -42,6 +45,30 @@ int l2_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3))
         int rc_ = (call);       \
         if (rc_ != L2_OK) return rc_; \
     } while (0)
+
+// A kernel's dynamic-LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize), raised when a launch needs more than it
+// was last raised to.  One of these per kernel (a function-local static at the launch site).  The attribute belongs to
+// the kernel as loaded on ONE device, so what was raised is kept per device; model handles on different host threads
+// share the launch sites, so the slow path is behind a mutex and the fast path reads an atomic.
+struct LdsLimit {
+    static constexpr int kMaxDevices = 64;
+    std::atomic<size_t> raised[kMaxDevices];
+    std::mutex mu;
+    explicit LdsLimit(size_t initial = 0) {
+        for (auto &r : raised) r.store(initial, std::memory_order_relaxed);
+    }
+    int ensure(const void *kernel, size_t bytes) {
+        int dev = 0;
+        L2_HIP(hipGetDevice(&dev));
+        if (dev < 0 || dev >= kMaxDevices) return l2_fail(L2_ERR_HIP, "device %d: more devices than the launch tables hold", dev);
+        if (bytes <= raised[dev].load(std::memory_order_acquire)) return L2_OK;
+        std::lock_guard<std::mutex> lock(mu);
+        if (bytes <= raised[dev].load(std::memory_order_relaxed)) return L2_OK;
+        L2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        raised[dev].store(bytes, std::memory_order_release);
+        return L2_OK;
+    }
+};
 
 // Position at which the prefill ladder 64/32/16/8/4/2 (src/inference.rs:78-127) leaves off.
 int l2_prefill_ladder_end(int n_prompt);
@@ -100,6 +127,11 @@ struct Q4Launch {
     float eps;   // rmsnorm epsilon, used when wn is set
     int rows_per_block; // filled by the streaming launcher
 };
+// The launch description travels by value as the kernel's one argument: it must stay far inside the 4 KB a
+// dispatch packet's argument block holds, and be plain data that a byte copy reproduces.
+static_assert(sizeof(Q4Launch) <= 1024, "Q4Launch is passed by value as a kernel argument");
+static_assert(std::is_trivially_copyable<Q4Launch>::value && std::is_standard_layout<Q4Launch>::value,
+              "Q4Launch is copied byte for byte into the dispatch's argument block");
 
 // When armed (profiling runs only), the next q4 launch goes out through
 // hipExtLaunchKernel with these events, which then carry the dispatch's own
@@ -116,6 +148,8 @@ struct Q4NameHook {
     char *buf = nullptr;
     int cap = 0;
     bool armed = false;
+    int grid = 0, block = 0, rows_per_block = 0; // what the launch would have been
+    size_t lds = 0;
 };
 extern thread_local Q4NameHook g_q4_name;
 

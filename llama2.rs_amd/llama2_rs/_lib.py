@@ -92,6 +92,7 @@ SIGNATURES = {
     "l2_kernel_class_count": (_I, []),
     "l2_kernel_class_name": (C.c_char_p, [_I]),
     "l2_decode_profile": (_I, [_VP, _VP, C.c_int32, C.c_int32, _I, _VP, _VP]),
+    "l2_q4_plan": (_I, [_I, _VP, _I, _I, _I, _I, C.c_char_p, _SZ, _VP]),
     "l2_copy_bench": (_I, [_SZ, _I, C.POINTER(C.c_float)]),
 }
 

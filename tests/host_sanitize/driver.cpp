@@ -72,6 +72,38 @@ int main(int argc, char **argv) {
     l2_tokenizer_free(nullptr);
     l2_random_free(nullptr);
 
+    // the q4 launcher's planning and argument building for every decode launch of the three presets (no device,
+    // nothing launched): kernel chosen, grid within one round of two blocks per CU, LDS within the CU's 160 KB
+    {
+        struct Shape { const char *what; int in, n, out[3], g, pair, norm; };
+        const Shape shapes[] = {
+            {"7B q|k|v", 4096, 3, {4096, 4096, 4096}, 128, 0, 1},   {"7B wo", 4096, 1, {4096, 0, 0}, 128, 0, 0},
+            {"7B w1|w3", 4096, 2, {11008, 11008, 0}, 128, 1, 1},    {"7B w2", 11008, 1, {4096, 0, 0}, 128, 0, 0},
+            {"13B q|k|v", 5120, 3, {5120, 5120, 5120}, 128, 0, 1},  {"13B wo", 5120, 1, {5120, 0, 0}, 128, 0, 0},
+            {"13B w1|w3", 5120, 2, {13824, 13824, 0}, 128, 1, 1},   {"13B w2", 13824, 1, {5120, 0, 0}, 128, 0, 0},
+            {"70B q|k|v", 8192, 3, {8192, 1024, 1024}, 64, 0, 1},   {"70B wo", 8192, 1, {8192, 0, 0}, 64, 0, 0},
+            {"70B w1|w3", 8192, 2, {28672, 28672, 0}, 64, 1, 1},    {"70B w2", 28672, 1, {8192, 0, 0}, 64, 0, 0},
+            {"ragged", 4160, 1, {72, 0, 0}, 32, 0, 0},              {"tiny", 256, 2, {64, 8, 0}, 32, 0, 1},
+        };
+        for (const Shape &sh : shapes) {
+            char name[160];
+            int32_t geo[4] = {0, 0, 0, 0};
+            if (l2_q4_plan(sh.in, sh.out, sh.n, sh.g, sh.pair, sh.norm, name, sizeof name, geo) != L2_OK) {
+                fprintf(stderr, "%s: %s\n", sh.what, l2_last_error());
+                return 1;
+            }
+            REQUIRE(strlen(name) > 8);
+            REQUIRE(geo[0] >= 1 && geo[0] <= 4 * 256 && geo[1] >= 64 && geo[1] <= 1024 && geo[2] >= 1);
+            REQUIRE(geo[3] >= 0 && geo[3] <= 152 * 1024);
+        }
+        char name[8];
+        int32_t geo[4];
+        const int32_t bad_out[3] = {12, 0, 0};
+        REQUIRE(l2_q4_plan(4096, bad_out, 1, 128, 0, 0, name, sizeof name, geo) != L2_OK);   // out not a multiple of 8
+        REQUIRE(l2_q4_plan(4100, shapes[1].out, 1, 128, 0, 0, name, sizeof name, geo) != L2_OK);
+        REQUIRE(l2_q4_plan(4096, shapes[1].out, 4, 128, 0, 0, name, sizeof name, geo) != L2_OK);
+    }
+
     // tokenizer (src/tokenizer.rs:22-108): every token, round trips, buffers that are too small
     l2_tokenizer *tk = nullptr;
     REQUIRE(l2_tokenizer_open("/nonexistent/tokenizer.bin", 32000, &tk) != L2_OK);

@@ -616,18 +616,33 @@ GQA8_G64 = ck.Dims(dim=1024, hidden_dim=1408, n_layers=2, n_heads=8, n_kv_heads=
                    seq_len=160, group_size=64)   # the 70B head geometry and group size, small
 
 
+def _with_seq(d, seq_len):
+    return ck.Dims(d.dim, d.hidden_dim, d.n_layers, d.n_heads, d.n_kv_heads, d.vocab_size, seq_len, d.group_size)
+
+
+_SMALL_QG2 = ck.Dims(dim=512, hidden_dim=768, n_layers=3, n_heads=4, n_kv_heads=2, vocab_size=400, seq_len=0,
+                     group_size=128)
+_WIDE_7B = ck.Dims(dim=4096, hidden_dim=11008, n_layers=2, n_heads=32, n_kv_heads=32, vocab_size=320, seq_len=0,
+                   group_size=128)   # the 7B widths (BASELINE config 2 runs through this path), two layers
+
+
 @pytest.mark.parametrize("mode", ["mfma", "fp32"])
-@pytest.mark.parametrize("n,chunk", [(512, 128), (300, 128), (257, 64), (40, 64), (9, 2)],
-                         ids=["four_chunks", "short_last_chunk", "one_token_left", "one_short_chunk", "chunks_of_2"])
-def test_prefill_chunks_equals_chunk_by_chunk(ops, n, chunk, mode):
+@pytest.mark.parametrize("geom,n,chunk", [
+    (_SMALL_QG2, 512, 128), (_SMALL_QG2, 300, 128), (_SMALL_QG2, 257, 64), (_SMALL_QG2, 40, 64), (_SMALL_QG2, 9, 2),
+    (GQA8_G64, 300, 128), (MID, 300, 128), (_WIDE_7B, 300, 128)],
+    ids=["four_chunks", "short_last_chunk", "one_token_left", "one_short_chunk", "chunks_of_2",
+         "gqa8_g64_300_by_128", "qg4_g32_300_by_128", "7b_wide_300_by_128"])
+def test_prefill_chunks_equals_chunk_by_chunk(ops, geom, n, chunk, mode):
     """prefill<A> over a whole prompt (src/inference.rs:16-40) through l2_prefill_chunks, whose chunks overlap on
     two streams in the matrix-core mode, against the same chunks given to transformer<B> one by one: every cache
-    row of every layer and the logits that follow, bit for bit (the kernels and their operands are the same)."""
+    row of every layer and the logits that follow, bit for bit (the kernels and their operands are the same).
+    Geometries: 2, 4 and 8 query heads per kv head, groups of 32, 64 and 128, and the 7B widths."""
     from llama2_rs import _lib
     from llama2_rs._lib import L2Error
-    dims = ck.Dims(dim=512, hidden_dim=768, n_layers=3, n_heads=4, n_kv_heads=2, vocab_size=400, seq_len=n + 8,
-                   group_size=128)
-    img = ck.synth_weights_image(dims, seed=11)
+    if geom is _WIDE_7B and mode == "fp32":
+        pytest.skip("the fp32 mode runs on one stream: covered by the small geometries")
+    dims = _with_seq(geom, n + 8)
+    img = ops.synth_image(dims, 11) if geom is _WIDE_7B else ck.synth_weights_image(dims, seed=11)
     m = ops.Model(img, dims)
     m.set_prefill_mode(_lib.PREFILL_MFMA if mode == "mfma" else _lib.PREFILL_FP32)
     rng = np.random.default_rng(n)

@@ -18,6 +18,17 @@ class _Hip:
         self.rt.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
         self.rt.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         self.rt.hipFree.argtypes = [C.c_void_p]
+        self.rt.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.rt.hipStreamDestroy.argtypes = [C.c_void_p]
+        self.rt.hipStreamSynchronize.argtypes = [C.c_void_p]
+        self.rt.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        self.rt.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        self.rt.hipGraphGetNodes.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_size_t)]
+        self.rt.hipGraphNodeGetType.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
+        self.rt.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        self.rt.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        self.rt.hipGraphDestroy.argtypes = [C.c_void_p]
         self.bufs = []
 
     def upload(self, a: np.ndarray) -> int:
@@ -74,4 +85,52 @@ def test_matvec_without_allocation_equals_the_allocating_entry_point():
     np.testing.assert_array_equal(hip.download(y1, want1.shape), want1)
     big.close()
     small.close()
+    hip.close()
+
+
+def test_matvec_without_allocation_under_graph_capture():
+    """The first call on a handle made while the stream is being captured (the handle's creation has done what a
+    first launch does besides enqueueing), no memset node in the graph, and every replay — with eager work of the
+    same operator and synchronisations between the replays — equal to the allocating entry point, bit for bit."""
+    from llama2_rs import ops, _lib
+    assert _lib.lib().l2_device_count() >= 1, "no HIP device: the GPU tests cannot run"
+    hip = _Hip()
+    rt = hip.rt
+    rng = np.random.default_rng(1)
+    q = ops.QLinear(*ck.synth_qlinear(rng, 4096, 512, 128, act_order=True), 128)
+    other = ops.QLinear(*ck.synth_qlinear(rng, 1024, 264, 64, act_order=True), 64)
+    xs = [rng.standard_normal((2, 4096)).astype(np.float32) for _ in range(3)]
+    want = [q.matvec(x) for x in xs]
+    dx, dy = hip.upload(xs[0]), hip.empty(want[0].nbytes)
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert rt.hipStreamCreate(C.byref(stream)) == 0
+    assert rt.hipStreamBeginCapture(stream, 0) == 0            # hipStreamCaptureModeGlobal
+    try:
+        q.matvec_device(dx, 2, dy, stream=stream.value)        # the handle's first device call: under capture
+    finally:
+        assert rt.hipStreamEndCapture(stream, C.byref(graph)) == 0
+    n_nodes = C.c_size_t()
+    assert rt.hipGraphGetNodes(graph, None, C.byref(n_nodes)) == 0 and n_nodes.value >= 2
+    nodes = (C.c_void_p * n_nodes.value)()
+    assert rt.hipGraphGetNodes(graph, nodes, C.byref(n_nodes)) == 0
+    for node in nodes:
+        kind = C.c_int()
+        assert rt.hipGraphNodeGetType(C.c_void_p(node), C.byref(kind)) == 0
+        assert kind.value == 0, f"graph node of type {kind.value}: only kernel nodes are expected"   # hipGraphNodeTypeKernel
+    assert rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+    for x, w in zip(xs, want):
+        assert rt.hipMemcpy(C.c_void_p(dx), x.ctypes.data_as(C.c_void_p), x.nbytes, 1) == 0
+        assert rt.hipGraphLaunch(gexec, stream) == 0
+        assert rt.hipStreamSynchronize(stream) == 0
+        np.testing.assert_array_equal(hip.download(dy, w.shape), w)
+        # eager work on the shared scratch between the replays
+        x2 = rng.standard_normal((3, 1024)).astype(np.float32)
+        d2, y2 = hip.upload(x2), hip.empty(3 * 264 * 4)
+        other.matvec_device(d2, 3, y2)
+        np.testing.assert_array_equal(hip.download(y2, (3, 264)), other.matvec(x2))
+    assert rt.hipGraphExecDestroy(gexec) == 0
+    assert rt.hipGraphDestroy(graph) == 0
+    assert rt.hipStreamDestroy(stream) == 0
+    q.close()
+    other.close()
     hip.close()
