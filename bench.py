@@ -305,7 +305,7 @@ def decode_run(np, M: Loaded, W: int, K: int, pos0: int, cpu: bool, cpu_tokens: 
     return out
 
 
-def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool) -> dict:
+def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool, cpu_tokens: int = 0) -> dict:
     """BASELINE config 2: a prompt of n random ids prefilled in chunks through the dequant->fp16 MFMA GEMM path,
     followed by K greedy decode steps."""
     from llama2_rs import _lib
@@ -337,6 +337,28 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool) -
         ids32, _ = m.decode_bench(int(prompt[-1]), n, K)
         out["fp32_path_tok_s"] = round(n / t_fp32, 1)
         out["greedy_tokens_same_as_after_fp32_prefill"] = f"{int(np.sum(np.cumprod(ids == ids32)))}/{K}"
+    if cpu_tokens > 0:
+        # the CPU restatement's fp32 prefill of the same prompt (chunks of 64, as the reference's ladder starts) and
+        # its B=1 loop: the first cpu_tokens greedy tokens against the GPU's after the MFMA prefill
+        from oracle import oracle_lib
+        o = oracle_lib.Model(M.img, d, max_seq=M.max_seq)
+        o.new_state()
+        toks = np.concatenate([[1], prompt[:n - 1]]).astype(np.int32)
+        t0 = time.perf_counter()
+        for c0 in range(0, n, 64):
+            c1 = min(c0 + 64, n)
+            o.transformer(toks[c0:c1], np.arange(c0, c1, dtype=np.int32))
+        t_cpu_prefill = time.perf_counter() - t0
+        tokc, cpu_ids = int(prompt[-1]), []
+        for i in range(min(cpu_tokens, K)):
+            tokc = oracle_lib.argmax(o.transformer([tokc], [n + i]))
+            cpu_ids.append(tokc)
+        same = int(np.sum(np.cumprod(np.asarray(cpu_ids) == ids[:len(cpu_ids)])))
+        out["greedy_tokens_identical_to_cpu"] = f"{same}/{len(cpu_ids)}"
+        out["cpu_baseline"] = {"value": round(n / t_cpu_prefill, 1), "unit": "tok/s", "cores": oracle_lib.num_threads(), "kind": "port",
+                               "sample": f"C restatement of the reference CPU path: fp32 prefill of the same {n}-token prompt in "
+                                         f"chunks of 64 (prefill<64>), then {len(cpu_ids)} greedy tokens for the comparison"}
+        o.close()
     m.set_prefill_mode(_lib.PREFILL_FP32)
     tok_s = n / t_mfma
     tflops = flops_per_token * tok_s / 1e12
@@ -400,6 +422,7 @@ def main() -> int:
     from llama2_rs import ops
 
     if a.workload == "matvec":
+        ops.copy_bench(1 << 28, 8)   # the plain copy of known size that counter readings of this run are scaled by
         r = matvec_run(np, ops, a.instances, a.iters, 5, not a.no_cpu_baseline)
         result = {"metric": "GPTQ matvec HBM GB/s (% of peak) on 1 MI355X", "value": r["value"], "unit": "GB/s", "n_gpus": 1,
                   "steps": r["steps"], "warmup": r["warmup"], "ms_per_step": r["ms_per_step"], "higher_is_better": True,
@@ -448,7 +471,8 @@ def main() -> int:
         if 1 in want:   # config 1 at its stated length
             configs["cfg1_7B_decode_16+256"] = decode_run(np, M, 16, 256, 0, False, 0)
         if 2 in want:   # config 2: 512-token prompt in chunks of 128 through the MFMA path, then 64 greedy steps
-            configs["cfg2_7B_prefill_512_by_128"] = prefill_run(np, M, 512, 128, 64, False)
+            configs["cfg2_7B_prefill_512_by_128"] = prefill_run(np, M, 512, 128, 64, False,
+                                                                 0 if a.no_cpu_baseline else 16)
         M.close()
         if 3 in want:
             M3 = Loaded(ops, "13B", 0, 0, 32 + 256 + 16, a.seed)

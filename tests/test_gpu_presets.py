@@ -243,3 +243,41 @@ def test_7b_full_depth_prefill_512_mfma_then_64_greedy(ops, oracle):
     assert same >= 8, (same, ids[:same + 1], ref[:same + 1])
     m.close()
     o.close()
+
+
+def test_70b_full_depth_greedy_behind_4096_positions(ops, oracle):
+    """BASELINE config 4 at full depth: the Llama-2-70B architecture in full (80 layers, 64 query / 8 kv heads,
+    group 64, 41 GB of weights), the cache pre-filled to 4096 positions (synthetic rows written on the device and
+    copied into the oracle's cache), then greedy tokens through the B=1 loop with the argmax fed back on the device,
+    against the oracle's loop: logits of the first position within 1e-4, 16 tokens identical (the CPU path takes
+    more than a second per token at this size), the last layer's new cache rows within 1e-4."""
+    dims = ops.preset("70B", 64)
+    ctx, n = 4096, 16
+    img = ops.synth_image(dims, 0)
+    m = ops.Model(img, dims, max_seq=ctx + n + 8)
+    o = oracle.Model(img, dims, max_seq=ctx + n + 8)
+    m.reset()
+    o.new_state()
+    m.fill_kv_synthetic(0, ctx, seed=1)
+    ko, vo = o.kv_cache()
+    for l in range(dims.n_layers):
+        k, v = m.read_kv(l, 0, ctx)
+        ko[l, :ctx] = k
+        vo[l, :ctx] = v
+    tok = 17
+    ref = o.transformer([tok], [ctx])
+    out = m.forward([tok], [ctx])
+    assert nrel(out, ref) < REL_FP32
+    tok = oracle.argmax(ref)
+    assert int(np.argmax(out)) == tok
+    ids, _ = m.decode_bench(tok, ctx + 1, n - 1)
+    want = []
+    for pos in range(ctx + 1, ctx + n):
+        tok = oracle.argmax(o.transformer([tok], [pos]))
+        want.append(tok)
+    np.testing.assert_array_equal(ids, want)
+    k, v = m.read_kv(dims.n_layers - 1, ctx, n)
+    assert nrel(k, ko[-1, ctx:ctx + n]) < REL_FP32
+    assert nrel(v, vo[-1, ctx:ctx + n]) < REL_FP32
+    m.close()
+    o.close()
