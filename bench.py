@@ -314,20 +314,27 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool, c
     prompt = rng.integers(0, d.vocab_size, size=n).astype(np.int32)
     flops_per_token = 2 * d.n_layers * (2 * d.dim * d.dim + 2 * d.dim * d.kv_dim + 3 * d.dim * d.hidden_dim)
 
+    reps, spread = 5, []
+
     def run(mode):
         m.set_prefill_mode(mode)
         m.reset()
-        m.forward(prompt[:min(chunk, n)], np.arange(min(chunk, n), dtype=np.int32))  # warm-up chunk
-        m.reset()
+        m.prefill_chunks(np.concatenate([[1], prompt[:n - 1]]).astype(np.int32), 0, chunk)   # untimed: the whole prompt once
         toks = np.concatenate([[1], prompt[:n - 1]]).astype(np.int32)  # START-shifted, as prefill<A> does
-        t0 = time.perf_counter()
-        if os.environ.get("L2_BENCH_PREFILL") == "serial":   # chunk by chunk through transformer<B>
-            for c0 in range(0, n, chunk):
-                c1 = min(c0 + chunk, n)
-                m.forward(toks[c0:c1], np.arange(c0, c1, dtype=np.int32))
-        else:
-            m.prefill_chunks(toks, 0, chunk)
-        return time.perf_counter() - t0
+        times = []
+        for _ in range(reps):   # the whole prompt each time, from an empty cache; the median is reported
+            m.reset()
+            t0 = time.perf_counter()
+            if os.environ.get("L2_BENCH_PREFILL") == "serial":   # chunk by chunk through transformer<B>
+                for c0 in range(0, n, chunk):
+                    c1 = min(c0 + chunk, n)
+                    m.forward(toks[c0:c1], np.arange(c0, c1, dtype=np.int32))
+            else:
+                m.prefill_chunks(toks, 0, chunk)
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        spread.append((times[0], times[-1]))
+        return times[len(times) // 2]
 
     t_mfma = run(_lib.PREFILL_MFMA)
     ids, ms_dec = m.decode_bench(int(prompt[-1]), n, K)
@@ -368,6 +375,7 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool, c
                     f"MFMA GEMM, then {K} greedy steps",
         "value": round(tok_s, 1), "unit": "tok/s", "steps": n_chunks, "warmup": 1,
         "ms_per_step": round(t_mfma * 1e3 / n_chunks, 3), "dtype": "f16 x f16 -> f32 (MFMA)",
+        "timing": f"one untimed prefill of the whole prompt, then the median of {reps} (fastest {n / spread[0][0]:.0f}, slowest {n / spread[0][1]:.0f} tok/s)",
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
                      "flops_per_token": flops_per_token},
