@@ -300,9 +300,12 @@ struct l2_model {
     size_t gemm_ws_floats = 0;
     int32_t *dtok = nullptr, *dpos = nullptr;
     unsigned long long *amax = nullptr;
-    // l2_prefill_chunks: a second stream with a second set of chunk buffers (consecutive chunks of a prompt run
-    // side by side, one layer apart), the whole prompt's ids and positions, one event per layer and stream
-    hipStream_t stream2 = nullptr;
+    // l2_prefill_chunks: further streams, each with a set of chunk buffers of its own (consecutive chunks of a
+    // prompt run side by side, one layer apart), the whole prompt's ids and positions, one event per layer and lane.
+    // Lane 0 is the model's stream with its primary buffers; lanes 1.. use extra[lane - 1].
+    static constexpr int kMaxLanes = 4; // the process has four hardware queues
+    int n_lanes = 2;
+    hipStream_t extra_stream[kMaxLanes - 1] = {nullptr, nullptr, nullptr};
     struct ChunkBufs {
         float *x = nullptr, *xq = nullptr, *xk = nullptr, *xv = nullptr, *qv = nullptr, *kv = nullptr, *vv = nullptr;
         void *h16a = nullptr, *h16b = nullptr, *h16c = nullptr;
@@ -310,11 +313,11 @@ struct l2_model {
         size_t gemm_ws_floats = 0;
         const int32_t *dtok = nullptr, *dpos = nullptr;
     };
-    ChunkBufs alt;
-    int cap_B_alt = 0;
+    ChunkBufs extra[kMaxLanes - 1];
+    int cap_B_extra[kMaxLanes - 1] = {0, 0, 0};
     int32_t *pf_tok = nullptr, *pf_pos = nullptr;
     int cap_pf = 0;
-    std::vector<hipEvent_t> pf_ev[2];
+    std::vector<hipEvent_t> pf_ev[kMaxLanes];
     hipEvent_t pf_join = nullptr;
     int32_t *dprompt = nullptr, *dout_ids = nullptr;
     int cap_prompt = 0, cap_out = 0;
@@ -477,6 +480,10 @@ static int model_build(const char *weights, size_t nbytes, const l2_dims *dims, 
 
     l2_model *m = new l2_model();
     m->use_graph = getenv("L2_STEP_GRAPH") != nullptr; // also l2_model_set_step_graph
+    if (const char *v = getenv("L2_PREFILL_LANES")) { // chunks of a prompt in flight at once (l2_prefill_chunks)
+        const int n = atoi(v);
+        if (n >= 1 && n <= l2_model::kMaxLanes) m->n_lanes = n;
+    }
     m->d = *dims;
     m->max_seq = max_seq;
     m->head_size = dims->dim / dims->n_heads;
@@ -680,19 +687,24 @@ extern "C" int l2_model_open(const char *path, const l2_dims *expect, int max_se
 extern "C" void l2_model_close(l2_model *m) {
     if (!m) return;
     if (m->stream) (void)hipStreamSynchronize(m->stream);
+    for (hipStream_t es : m->extra_stream)
+        if (es) (void)hipStreamSynchronize(es);
     void *ptrs[] = {m->dimage, m->dinv, m->rope_cos, m->rope_sin, m->dwn, m->attn_part, m->x, m->xq, m->xk,
                     m->xv, m->qv, m->kv, m->vv, m->attg, m->x1, m->x3, m->hg, m->hd, m->logits, m->dtok, m->dpos, m->dloop,
                     m->amax, m->dprompt, m->dout_ids, m->op_x, m->op_xg, m->op_y, m->h16a, m->h16b, m->h16c,
                     m->hb, m->hb2, m->ssb, m->gemm_ws};
     for (void *p : ptrs) dfree(p);
-    if (m->stream2) (void)hipStreamSynchronize(m->stream2);
-    void *alts[] = {m->alt.x, m->alt.xq, m->alt.xk, m->alt.xv, m->alt.qv, m->alt.kv, m->alt.vv, m->alt.h16a, m->alt.h16b,
-                    m->alt.h16c, m->alt.hb, m->alt.hb2, m->alt.ssb, m->alt.gemm_ws, m->pf_tok, m->pf_pos};
-    for (void *p : alts) dfree(p);
+    for (auto &a : m->extra) {
+        void *bufs[] = {a.x, a.xq, a.xk, a.xv, a.qv, a.kv, a.vv, a.h16a, a.h16b, a.h16c, a.hb, a.hb2, a.ssb, a.gemm_ws};
+        for (void *p : bufs) dfree(p);
+    }
+    dfree(m->pf_tok);
+    dfree(m->pf_pos);
     for (auto &v : m->pf_ev)
         for (hipEvent_t e : v) (void)hipEventDestroy(e);
     if (m->pf_join) (void)hipEventDestroy(m->pf_join);
-    if (m->stream2) (void)hipStreamDestroy(m->stream2);
+    for (hipStream_t es : m->extra_stream)
+        if (es) (void)hipStreamDestroy(es);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
@@ -740,7 +752,8 @@ static int ensure_batch_mfma(l2_model *m, int B);
 // Nothing may be running on either of the model's streams when a buffer they use is freed.
 static int drain_streams(l2_model *m) {
     L2_HIP(hipStreamSynchronize(m->stream));
-    if (m->stream2) L2_HIP(hipStreamSynchronize(m->stream2));
+    for (hipStream_t es : m->extra_stream)
+        if (es) L2_HIP(hipStreamSynchronize(es));
     return L2_OK;
 }
 
@@ -1343,9 +1356,9 @@ static l2_model::ChunkBufs primary_bufs(const l2_model *m) {
 }
 
 // The chunk's buffers and stream are arguments: l2_prefill_chunks runs consecutive chunks on two streams.  What a
-// chunk needs from the one before it is that chunk's cache rows of the same layer, so `after_kv[l]` is recorded
-// behind the kernel that writes this chunk's rows of layer l and `before_attn[l]` is waited for in front of the
-// attention of layer l (either may be null).
+// chunk needs from the ones before it is their cache rows of the same layer, so `before_attn[l]` (the event of the
+// chunk before) is waited for in front of the attention of layer l, behind the kernel that writes this chunk's own
+// rows of layer l, and `after_kv[l]` is recorded right there (either may be null).
 static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos, const l2_model::ChunkBufs &b,
                                 hipStream_t st, const hipEvent_t *after_kv, const hipEvent_t *before_attn) {
     L2_TRY(check_position(m, max_pos));
@@ -1386,8 +1399,11 @@ static int forward_enqueue_mfma(l2_model *m, l2_state *s, int B, int max_pos, co
         R.ws = b.gemm_ws, R.B = B, R.ss = b.ssb, R.pos = b.dpos, R.cos_t = m->rope_cos, R.sin_t = m->rope_sin;
         R.q = b.qv, R.kcache = kc, R.vcache = vc, R.n_heads = d.n_heads, R.n_kv_heads = d.n_kv_heads;
         L2_TRY(gemm_rope_kv_launch(R, st));
-        if (after_kv) L2_HIP(hipEventRecord(after_kv[l], st));
+        // Wait first, record second: the event of this chunk then stands for its own rows of layer l AND, through
+        // the event it waited for, for those of every chunk before it, so that a chunk two or more lanes behind
+        // needs to wait for its direct predecessor only.
         if (before_attn) L2_HIP(hipStreamWaitEvent(st, before_attn[l], 0));
+        if (after_kv) L2_HIP(hipEventRecord(after_kv[l], st));
         L2_TRY(attention_launch(nullptr, b.h16a, b.qv, kc, vc, b.dpos, wo.inv_index, d.n_heads, d.n_kv_heads,
                                 m->head_size, max_pos, B, st));
         {   // wo: partial tiles, then residual + rms scale + the fp16 inputs of w1 and w3 in one kernel
@@ -1474,63 +1490,66 @@ extern "C" int l2_forward(l2_model *m, l2_state *s, const int32_t *tokens, const
 
 // The second set of chunk buffers, the second stream and the per-layer events of l2_prefill_chunks.
 static int ensure_prefill_pipeline(l2_model *m, int B, int n) {
-    if (!m->stream2) L2_HIP(hipStreamCreate(&m->stream2)); // default priority, as the model's own
+    const int lanes = B > 0 ? m->n_lanes : 1;
+    for (int i = 0; i + 1 < lanes; i++)
+        if (!m->extra_stream[i]) L2_HIP(hipStreamCreate(&m->extra_stream[i])); // default priority, as the model's own
     if (!m->pf_join) L2_HIP(hipEventCreateWithFlags(&m->pf_join, hipEventDisableTiming));
-    for (auto &v : m->pf_ev)
-        while ((int)v.size() < m->d.n_layers) {
+    for (int i = 0; i < lanes; i++)
+        while ((int)m->pf_ev[i].size() < m->d.n_layers) {
             hipEvent_t e = nullptr;
             L2_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-            v.push_back(e);
+            m->pf_ev[i].push_back(e);
         }
     if (n > m->cap_pf) {
-        L2_HIP(hipStreamSynchronize(m->stream));
-        L2_HIP(hipStreamSynchronize(m->stream2));
+        L2_TRY(drain_streams(m));
         dfree(m->pf_tok), dfree(m->pf_pos);
         m->pf_tok = m->pf_pos = nullptr, m->cap_pf = 0;
         L2_TRY(dalloc(&m->pf_tok, (size_t)n));
         L2_TRY(dalloc(&m->pf_pos, (size_t)n));
         m->cap_pf = n;
     }
-    if (B <= m->cap_B_alt) return L2_OK;
-    L2_TRY(drain_streams(m));
-    l2_model::ChunkBufs &a = m->alt;
-    void **bufs[] = {(void **)&a.x, (void **)&a.xq, (void **)&a.xk, (void **)&a.xv, (void **)&a.qv, (void **)&a.kv,
-                     (void **)&a.vv, &a.h16a, &a.h16b, &a.h16c, (void **)&a.hb, (void **)&a.hb2, (void **)&a.ssb,
-                     (void **)&a.gemm_ws};
-    for (void **b : bufs) {
-        dfree(*b);
-        *b = nullptr;
+    for (int i = 0; i + 1 < lanes; i++) {
+        if (B <= m->cap_B_extra[i]) continue;
+        L2_TRY(drain_streams(m));
+        l2_model::ChunkBufs &a = m->extra[i];
+        void **bufs[] = {(void **)&a.x, (void **)&a.xq, (void **)&a.xk, (void **)&a.xv, (void **)&a.qv, (void **)&a.kv,
+                         (void **)&a.vv, &a.h16a, &a.h16b, &a.h16c, (void **)&a.hb, (void **)&a.hb2, (void **)&a.ssb,
+                         (void **)&a.gemm_ws};
+        for (void **b : bufs) {
+            dfree(*b);
+            *b = nullptr;
+        }
+        m->cap_B_extra[i] = 0;
+        const size_t dim = m->d.dim, hid = m->d.hidden_dim, kvd = m->kv_dim, wide = std::max(dim, hid);
+        L2_TRY(dalloc(&a.x, B * dim));
+        L2_TRY(dalloc(&a.xq, B * dim));
+        L2_TRY(dalloc(&a.xk, B * dim));
+        L2_TRY(dalloc(&a.xv, B * dim));
+        L2_TRY(dalloc(&a.qv, B * dim));
+        L2_TRY(dalloc(&a.kv, B * kvd));
+        L2_TRY(dalloc(&a.vv, B * kvd));
+        uint16_t *h = nullptr;
+        L2_TRY(dalloc(&h, B * wide));
+        a.h16a = h;
+        L2_TRY(dalloc(&h, B * wide));
+        a.h16b = h;
+        L2_TRY(dalloc(&h, B * wide));
+        a.h16c = h;
+        L2_TRY(dalloc(&a.hb, B * hid));
+        L2_TRY(dalloc(&a.hb2, B * hid));
+        L2_TRY(dalloc(&a.ssb, (size_t)B));
+        a.gemm_ws_floats = (size_t)8 * B * std::max((size_t)2 * hid, dim + 2 * kvd) / 2;
+        L2_TRY(dalloc(&a.gemm_ws, a.gemm_ws_floats));
+        m->cap_B_extra[i] = B;
     }
-    m->cap_B_alt = 0;
-    const size_t dim = m->d.dim, hid = m->d.hidden_dim, kvd = m->kv_dim, wide = std::max(dim, hid);
-    L2_TRY(dalloc(&a.x, B * dim));
-    L2_TRY(dalloc(&a.xq, B * dim));
-    L2_TRY(dalloc(&a.xk, B * dim));
-    L2_TRY(dalloc(&a.xv, B * dim));
-    L2_TRY(dalloc(&a.qv, B * dim));
-    L2_TRY(dalloc(&a.kv, B * kvd));
-    L2_TRY(dalloc(&a.vv, B * kvd));
-    uint16_t *h = nullptr;
-    L2_TRY(dalloc(&h, B * wide));
-    a.h16a = h;
-    L2_TRY(dalloc(&h, B * wide));
-    a.h16b = h;
-    L2_TRY(dalloc(&h, B * wide));
-    a.h16c = h;
-    L2_TRY(dalloc(&a.hb, B * hid));
-    L2_TRY(dalloc(&a.hb2, B * hid));
-    L2_TRY(dalloc(&a.ssb, (size_t)B));
-    a.gemm_ws_floats = (size_t)8 * B * std::max((size_t)2 * hid, dim + 2 * kvd) / 2;
-    L2_TRY(dalloc(&a.gemm_ws, a.gemm_ws_floats));
-    m->cap_B_alt = B;
     return L2_OK;
 }
 
 // prefill<A> (src/inference.rs:16-40) for a whole prompt: tokens[i] at position pos0 + i, in chunks of `chunk`,
-// no logits.  With the matrix-core mode consecutive chunks run on two streams, each with buffers of its own:
+// no logits.  With the matrix-core mode consecutive chunks run on n_lanes streams, each with buffers of its own:
 // a chunk needs from its predecessor only that chunk's cache rows of the same layer (an event per layer), so
-// the second chunk follows one layer behind the first and its kernels fill the compute units that the first
-// one's short launches leave idle.  The arithmetic of a chunk is that of l2_forward on the same chunk.
+// every chunk follows one layer behind the one before it and its kernels fill the compute units that the
+// others' short launches leave idle.  The arithmetic of a chunk is that of l2_forward on the same chunk.
 extern "C" int l2_prefill_chunks(l2_model *m, l2_state *s, const int32_t *tokens, int n, int pos0, int chunk) {
     if (!m || !s || !tokens) return l2_fail(L2_ERR_ARG, "null argument");
     if (s->m != m) return l2_fail(L2_ERR_ARG, "state belongs to another model");
@@ -1553,32 +1572,36 @@ extern "C" int l2_prefill_chunks(l2_model *m, l2_state *s, const int32_t *tokens
     L2_HIP(hipMemcpy(m->pf_pos, pos.data(), (size_t)n * 4, hipMemcpyHostToDevice));
     // Everything that is enqueued on the two streams; a failure half-way returns through the caller below, which
     // first waits for what earlier chunks already have in flight on either stream.
+    const int lanes = mfma ? m->n_lanes : 1;
+    // the model's stream waits for everything the other lanes have been given so far
+    auto join_lanes = [&]() -> int {
+        for (int i = 0; i + 1 < lanes; i++) {
+            L2_HIP(hipEventRecord(m->pf_join, m->extra_stream[i]));
+            L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
+        }
+        return L2_OK;
+    };
     auto enqueue_all = [&]() -> int {
         int c = 0;
         for (int c0 = 0; c0 < n; c0 += chunk, c++) {
             const int B = std::min(chunk, n - c0);
             const int max_pos = pos0 + c0 + B - 1;
             if (mfma && B > 1) {
-                l2_model::ChunkBufs b = (c & 1) ? m->alt : primary_bufs(m);
+                const int lane = c % lanes, before = (c + lanes - 1) % lanes;
+                l2_model::ChunkBufs b = lane ? m->extra[lane - 1] : primary_bufs(m);
                 b.dtok = m->pf_tok + c0, b.dpos = m->pf_pos + c0;
-                hipStream_t st = (c & 1) ? m->stream2 : m->stream;
-                L2_TRY(forward_enqueue_mfma(m, s, B, max_pos, b, st, m->pf_ev[c & 1].data(),
-                                            c > 0 ? m->pf_ev[(c - 1) & 1].data() : nullptr));
+                hipStream_t st = lane ? m->extra_stream[lane - 1] : m->stream;
+                L2_TRY(forward_enqueue_mfma(m, s, B, max_pos, b, st, m->pf_ev[lane].data(),
+                                            c > 0 ? m->pf_ev[before].data() : nullptr));
             } else {
                 // one token left over, or the fp32 mode: the fp32 kernels on the model's stream, behind everything
-                if (c > 0 && mfma) {
-                    L2_HIP(hipEventRecord(m->pf_join, m->stream2));
-                    L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
-                }
+                if (c > 0 && mfma) L2_TRY(join_lanes());
                 L2_HIP(hipMemcpyAsync(m->dtok, m->pf_tok + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
                 L2_HIP(hipMemcpyAsync(m->dpos, m->pf_pos + c0, (size_t)B * 4, hipMemcpyDeviceToDevice, m->stream));
                 L2_TRY(forward_enqueue(m, s, B, max_pos, false));
             }
         }
-        if (mfma) {
-            L2_HIP(hipEventRecord(m->pf_join, m->stream2));
-            L2_HIP(hipStreamWaitEvent(m->stream, m->pf_join, 0));
-        }
+        if (mfma) L2_TRY(join_lanes());
         return L2_OK;
     };
     const int rc = enqueue_all();
@@ -1589,7 +1612,8 @@ extern "C" int l2_prefill_chunks(l2_model *m, l2_state *s, const int32_t *tokens
         char keep[sizeof g_err];
         memcpy(keep, g_err, sizeof keep);
         (void)hipStreamSynchronize(m->stream);
-        if (m->stream2) (void)hipStreamSynchronize(m->stream2);
+        for (hipStream_t es : m->extra_stream)
+            if (es) (void)hipStreamSynchronize(es);
         memcpy(g_err, keep, sizeof keep);
         return rc;
     }
