@@ -143,19 +143,20 @@ def matvec_run(np, ops, n_inst: int, iters: int, reps: int, cpu: bool) -> dict:
             traffic, note = t["FETCH_SIZE"][name] + t["WRITE_SIZE"][name], "profiles/q4_matvec_cfg0_hbm_counters.txt"
         else:
             note = f"profiles/q4_matvec_cfg0_hbm_counters.txt holds no reading for {name}: take it again"
-    gbs = nbytes / us_disp / 1e3
+    gbs = nbytes / us_cad / 1e3   # HIP events around the timed region on the launch stream, divided by its launches
     out = {
         "workload": (f"standalone GPTQ 4-bit act-order matvec, in {n_in}, out {n_out}, group {G}, batch 1; {n_inst} distinct "
                      f"weight instances ({n_inst * nbytes / 1e6:.0f} MB) launched round-robin, {iters} launches x {reps} runs"),
         "value": round(gbs, 1), "unit": "GB/s", "steps": iters, "warmup": n_inst,
-        "ms_per_step": round(us_disp * 1e-3, 6),
-        "us_per_launch_back_to_back": round(us_cad, 3),
-        "GBs_back_to_back": round(nbytes / us_cad / 1e3, 1),
+        "ms_per_step": round(us_cad * 1e-3, 6),
+        "us_per_dispatch_own_events": round(us_disp, 3),
+        "GBs_by_dispatch_events": round(nbytes / us_disp / 1e3, 1),
         "dtype": "f32",
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": note,
                      "algorithmic_bytes_per_launch": nbytes, "kernel": kernel,
-                     "duration": "mean of the dispatches' own start/stop events; back-to-back cadence beside it"},
+                     "duration": "HIP events around the timed launches on their stream, divided by the launches (median of the runs); "
+                                 "the mean of the dispatches' own start/stop events beside it"},
     }
     if cpu:
         from oracle import oracle_lib
