@@ -675,6 +675,50 @@ def test_prefill_chunks_equals_chunk_by_chunk(ops, geom, n, chunk, mode):
     m.close()
 
 
+_LANES_SNIPPET = r"""
+import sys, numpy as np
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[2])
+from llama2_rs import ops, _lib, checkpoint as ck
+n, chunk = 700, 128    # six chunks, the last one short: lanes are reused and their events recorded again
+dims = ck.Dims(dim=512, hidden_dim=768, n_layers=3, n_heads=4, n_kv_heads=2, vocab_size=400, seq_len=n + 8, group_size=128)
+m = ops.Model(ck.synth_weights_image(dims, seed=11), dims)
+m.set_prefill_mode(_lib.PREFILL_MFMA)
+toks = np.random.default_rng(n).integers(0, dims.vocab_size, size=n).astype(np.int32)
+bad = 0
+for rep in range(2):
+    m.reset()
+    for c0 in range(0, n, chunk):
+        c1 = min(c0 + chunk, n)
+        m.forward(toks[c0:c1], np.arange(c0, c1, dtype=np.int32))
+    want = [m.read_kv(l, 0, n) for l in range(dims.n_layers)], m.forward([5], [n])
+    m.reset()
+    m.prefill_chunks(toks, 0, chunk)
+    got = [m.read_kv(l, 0, n) for l in range(dims.n_layers)], m.forward([5], [n])
+    for l in range(dims.n_layers):
+        bad += int(not np.array_equal(got[0][l][0], want[0][l][0])) + int(not np.array_equal(got[0][l][1], want[0][l][1]))
+    bad += int(not np.array_equal(got[1], want[1]))
+m.close()
+print("BAD", bad)
+"""
+
+
+@pytest.mark.parametrize("lanes", [1, 3, 4])
+def test_prefill_chunks_on_other_numbers_of_lanes(lanes):
+    """L2_PREFILL_LANES chooses how many chunks of a prompt are in flight when the library is loaded (default 2).
+    With three or four lanes a chunk's rows are needed by chunks that never waited for it directly: the event of
+    a chunk is recorded behind its own wait, so it stands for every earlier chunk.  Same bit-for-bit comparison
+    with the chunks given to transformer<B> one by one, in a process of its own."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, L2_PREFILL_LANES=str(lanes))
+    r = subprocess.run([sys.executable, "-c", _LANES_SNIPPET, os.path.join(root, "llama2.rs_amd"), root],
+                       capture_output=True, text=True, env=env, timeout=150)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.strip().endswith("BAD 0"), r.stdout[-500:]
+
+
 @pytest.mark.parametrize("dims,B", [(TINY_GQA, 5), (MID, 33), (MID, 128), (TINY, 37), (GQA8_G64, 5), (GQA8_G64, 64),
                                     (GQA8_G64, 130)],
                          ids=["gqa_g128_b5", "g32_b33", "g32_b128", "mha_g64_b37", "gqa8_g64_b5", "gqa8_g64_b64",
