@@ -106,7 +106,9 @@ def counter_table(path: str) -> dict:
 def matvec_run(np, ops, n_inst: int, iters: int, reps: int, cpu: bool) -> dict:
     """BASELINE config 0: the standalone GPTQ 4-bit matvec at the 7B q_proj shape (in = out = 4096, group 128,
     act-order, batch 1), launched back to back over n_inst distinct weight instances (more bytes than the 256 MB
-    memory-side cache holds, so every launch streams its weights from HBM).  Instance 0 is config 0 itself (numpy
+    memory-side cache holds, so every launch streams its weights from HBM).  What is timed is the whole operator on
+    device-resident x in its natural order, the act-order permutation of x included (one launch: the kernel applies it
+    while it stages x).  Instance 0 is config 0 itself (numpy
     default_rng(0): AutoGPTQ-layout tensors through the exporter's transform, x ~ N(0,1)) and is checked against
     the CPU restatement; the others draw the same distributions in the `.bin` layout directly."""
     from llama2_rs import checkpoint as ck
@@ -145,7 +147,7 @@ def matvec_run(np, ops, n_inst: int, iters: int, reps: int, cpu: bool) -> dict:
             note = f"profiles/q4_matvec_cfg0_hbm_counters.txt holds no reading for {name}: take it again"
     gbs = nbytes / us_cad / 1e3   # HIP events around the timed region on the launch stream, divided by its launches
     out = {
-        "workload": (f"standalone GPTQ 4-bit act-order matvec, in {n_in}, out {n_out}, group {G}, batch 1; {n_inst} distinct "
+        "workload": (f"standalone GPTQ 4-bit act-order matvec (x in natural order -> y), in {n_in}, out {n_out}, group {G}, batch 1; {n_inst} distinct "
                      f"weight instances ({n_inst * nbytes / 1e6:.0f} MB) launched round-robin, {iters} launches x {reps} runs"),
         "value": round(gbs, 1), "unit": "GB/s", "steps": iters, "warmup": n_inst,
         "ms_per_step": round(us_cad * 1e-3, 6),

@@ -36,8 +36,12 @@ int l2_state_fill_synthetic(l2_state *s, int pos0, int npos, uint64_t seed);
 /* ---- timing ---------------------------------------------------------------- */
 
 /* Launch the B=1 matvec of qs[0..n) round-robin `iters` times on device-resident
- * random x (no host copies inside the timed region), timed with HIP events on
- * the launch stream.  *ms_total is the elapsed time of all iters launches. */
+ * random x in its natural order (no host copies inside the timed region): the
+ * whole operator, QLinear::matvec<1> with its act-order permutation of x
+ * (src/gptq.rs:99-122), one launch per matvec where the kernel applies the
+ * permutation itself (rows of up to 8192 inputs), else a gather and the matvec.
+ * Timed with HIP events on the launch stream: *ms_total is the elapsed time of
+ * all iters matvecs. */
 int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_total);
 
 /* The same launches, each carrying its own start/stop events (hipExtLaunchKernel): *ms_sum is the sum of the

@@ -909,6 +909,19 @@ static int q4_one(const DevQLinear &q, const float *xg, float *y, int B, hipStre
     return q4_matvec_launch(L, st);
 }
 
+// QLinear::matvec<B> on x in its natural order (src/gptq.rs:94-176, the act-order gather of :99-122 included):
+// one launch where the kernel can apply g_index itself, else a gather into xg_scratch and the matvec.
+static int q4_one_natural(const DevQLinear &q, const float *x, float *xg_scratch, float *y, int B, hipStream_t st) {
+    Q4Launch L = launch_of(q, B, 0.f);
+    L.m[0] = mat_of(q, x, nullptr, y);
+    if (q4_gathers_in_kernel(L)) {
+        L.m[0].gidx = q.inv_index;
+        return q4_matvec_launch(L, st);
+    }
+    L2_TRY(gather_launch(xg_scratch, x, q.g_index, q.in, B, st));
+    return q4_one(q, xg_scratch, y, B, st);
+}
+
 static int check_qlinear_shape(int in, int out, int g) {
     if (g != 32 && g != 64 && g != 128) return l2_fail(L2_ERR_ARG, "group size %d (32, 64 or 128)", g);
     if (in <= 0 || out <= 0 || in % 32 || in % g || out % 8)
@@ -927,8 +940,9 @@ static int qlinear_warm_up(l2_qlinear *q) {
     float *fixed = nullptr;
     L2_TRY(scratch_ptr(&fixed));
     L2_HIP(hipMemsetAsync(q->x, 0, (size_t)q->q.in * 4, q->stream));
+    L2_TRY(q4_one_natural(q->q, q->x, q->xg, q->y, 1, q->stream));   // the form l2_qlinear_matvec runs
     L2_TRY(gather_launch(q->xg, q->x, q->q.g_index, q->q.in, 1, q->stream));
-    L2_TRY(q4_one(q->q, q->xg, q->y, 1, q->stream));
+    L2_TRY(q4_one(q->q, q->xg, q->y, 1, q->stream));                 // the form l2_qlinear_matvec_device runs
     L2_HIP(hipStreamSynchronize(q->stream));
     return L2_OK;
 }
@@ -1006,8 +1020,7 @@ static int qlinear_scratch(l2_qlinear *q, int B) {
 static int matvec_host(const DevQLinear &q, float *dx, float *dxg, float *dy, const float *x_host, int B,
                        float *y_host, hipStream_t st) {
     L2_HIP(hipMemcpyAsync(dx, x_host, (size_t)B * q.in * 4, hipMemcpyHostToDevice, st));
-    L2_TRY(gather_launch(dxg, dx, q.g_index, q.in, B, st));
-    L2_TRY(q4_one(q, dxg, dy, B, st));
+    L2_TRY(q4_one_natural(q, dx, dxg, dy, B, st));
     L2_HIP(hipMemcpyAsync(y_host, dy, (size_t)B * q.out * 4, hipMemcpyDeviceToHost, st));
     L2_HIP(hipStreamSynchronize(st));
     return L2_OK;
@@ -1814,17 +1827,17 @@ extern "C" int l2_qlinear_bench(l2_qlinear **qs, int n, int iters, float *ms_tot
     for (int i = 0; i < n; i++) {
         if (!qs[i]) return l2_fail(L2_ERR_ARG, "null qlinear %d", i);
         L2_TRY(qlinear_scratch(qs[i], 1));
-        L2_TRY(fill_pattern_launch(qs[i]->xg, (size_t)qs[i]->q.in, 17 + i, st));
+        L2_TRY(fill_pattern_launch(qs[i]->x, (size_t)qs[i]->q.in, 17 + i, st));
     }
     hipEvent_t e0, e1;
     L2_HIP(hipEventCreate(&e0));
     L2_HIP(hipEventCreate(&e1));
-    for (int i = 0; i < n; i++) L2_TRY(q4_one(qs[i]->q, qs[i]->xg, qs[i]->y, 1, st)); // warm-up
+    for (int i = 0; i < n; i++) L2_TRY(q4_one_natural(qs[i]->q, qs[i]->x, qs[i]->xg, qs[i]->y, 1, st)); // warm-up
     L2_HIP(hipStreamSynchronize(st));
     L2_HIP(hipEventRecord(e0, st));
-    for (int it = 0; it < iters; it++) {
+    for (int it = 0; it < iters; it++) { // the whole operator: x in its natural order -> y, the act-order gather included
         l2_qlinear *q = qs[it % n];
-        L2_TRY(q4_one(q->q, q->xg, q->y, 1, st));
+        L2_TRY(q4_one_natural(q->q, q->x, q->xg, q->y, 1, st));
     }
     L2_HIP(hipEventRecord(e1, st));
     L2_HIP(hipEventSynchronize(e1));
@@ -1840,9 +1853,15 @@ extern "C" int l2_qlinear_bench_dispatch(l2_qlinear **qs, int n, int iters, floa
     for (int i = 0; i < n; i++) {
         if (!qs[i]) return l2_fail(L2_ERR_ARG, "null qlinear %d", i);
         L2_TRY(qlinear_scratch(qs[i], 1));
-        L2_TRY(fill_pattern_launch(qs[i]->xg, (size_t)qs[i]->q.in, 17 + i, st));
+        L2_TRY(fill_pattern_launch(qs[i]->x, (size_t)qs[i]->q.in, 17 + i, st));
     }
-    for (int i = 0; i < n; i++) L2_TRY(q4_one(qs[i]->q, qs[i]->xg, qs[i]->y, 1, st)); // warm-up
+    for (int i = 0; i < n; i++) {
+        Q4Launch probe = launch_of(qs[i]->q, 1, 0.f);
+        probe.m[0] = mat_of(qs[i]->q, qs[i]->x, nullptr, qs[i]->y);
+        if (!q4_gathers_in_kernel(probe))
+            return l2_fail(L2_ERR_ARG, "dispatch timing covers the one-launch form of the operator only (in=%d)", qs[i]->q.in);
+        L2_TRY(q4_one_natural(qs[i]->q, qs[i]->x, qs[i]->xg, qs[i]->y, 1, st)); // warm-up
+    }
     L2_HIP(hipStreamSynchronize(st));
     std::vector<hipEvent_t> ev((size_t)iters * 2, nullptr);
     int rc = L2_OK;
@@ -1854,7 +1873,7 @@ extern "C" int l2_qlinear_bench_dispatch(l2_qlinear **qs, int n, int iters, floa
         g_q4_prof.start = ev[2 * (size_t)it];
         g_q4_prof.stop = ev[2 * (size_t)it + 1];
         g_q4_prof.armed = true;
-        rc = q4_one(q->q, q->xg, q->y, 1, st);
+        rc = q4_one_natural(q->q, q->x, q->xg, q->y, 1, st);
         if (rc == L2_OK && g_q4_prof.armed) rc = l2_fail(L2_ERR_ARG, "this form of the kernel takes no dispatch events");
         g_q4_prof.armed = false;
         if (rc == L2_OK) launched++;
@@ -1881,6 +1900,7 @@ extern "C" int l2_qlinear_kernel(l2_qlinear *q, char *out, size_t cap) {
     const float *some = (const float *)q->bufs[2]; // only null / non-null matters for the choice of kernel
     Q4Launch L = launch_of(q->q, 1, 0.f);
     L.m[0] = mat_of(q->q, some, nullptr, nullptr);
+    if (q4_gathers_in_kernel(L)) L.m[0].gidx = q->q.inv_index;
     g_q4_name.buf = out;
     g_q4_name.cap = (int)cap;
     g_q4_name.armed = true;

@@ -284,6 +284,9 @@ int q4_matvec_launch(Q4Launch &L, hipStream_t stream) {
         const char *v = getenv("L2_Q4_IMPL");
         return (v && !strcmp(v, "tile")) ? 1 : 0;
     }();
+    for (int i = 0; i < L.n_mats; i++)
+        if (L.m[i].gidx && !q4_gathers_in_kernel(L))
+            return l2_fail(L2_ERR_ARG, "q4 matvec: this launch cannot gather x itself (in=%d, %d matrices)", L.in, L.n_mats);
     if (!impl_tile && q4_stream_supports(L)) return q4_stream_launch(L, stream);
     // Rows per wave: enough waves to cover 256 CUs several times over, more
     // rows per wave (less LDS traffic per weight byte) once there are plenty.

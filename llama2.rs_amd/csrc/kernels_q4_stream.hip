@@ -155,6 +155,7 @@ struct MatOps {
     const int32_t *qzeros;
     const float *scales;
     const float *x;
+    const int32_t *gidx;
     const float *wn;
     float *y;
     int out;
@@ -166,6 +167,7 @@ __device__ __forceinline__ MatOps mat_ops(const Q4Mat &M) {
     o.qzeros = pin_s(M.qzeros);
     o.scales = pin_s(M.scales);
     o.x = pin_s(M.x);
+    o.gidx = pin_s(M.gidx);
     o.wn = pin_s(M.wn);
     o.y = pin_s(M.y);
     o.out = pin_s(M.out);
@@ -182,9 +184,14 @@ struct RowData {
 // MODE 1: integer-dot inner loop, x staged and quantised in LDS.
 // MODE 2: fp32 inner loop, one matrix without rmsnorm: every wave loads its own slice of x (coalesced)
 //         and turns it into the per-lane chunks through LDS of its own; no barrier before the first row.
-template <int G, int NWK, int S, bool PAIR, int MODE, int P>
+// GATHER (MODE 0, one matrix, no rmsnorm): x arrives in its natural order and the kernel applies the act-order
+//         permutation itself, x[g_index[j]] (src/gptq.rs:99-122), for a caller with no producer to do it: x and the
+//         inverse of g_index are requested together and every element is written straight to its place in the
+//         staged chunks (the scatter a producer's epilogue would have done); the chunk sums are taken by the lanes.
+template <int G, int NWK, int S, bool PAIR, int MODE, int P, bool GATHER = false>
 __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L) {
     constexpr bool IDOT = MODE == 1, DIRECT = MODE == 2;
+    static_assert(!GATHER || (MODE == 0 && !PAIR), "the gathering form takes one matrix through the block-wide staging");
     static_assert(!(DIRECT && PAIR), "the direct form takes one matrix");
     constexpr int NM = PAIR ? 2 : 1;
     constexpr int NW = NWK * S;
@@ -277,6 +284,16 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
     // the staging of x (a cache hit) must not queue behind rows that come from HBM.
     StageRegs xr[DIRECT ? 1 : NM];
     float4 xd[DIRECT ? 8 : 1];
+    int4 gi[GATHER ? kStageBatch : 1];
+    if constexpr (GATHER) { // the first batch covers the whole vector (checked by the launcher)
+        const int n4 = in >> 2;
+        const int4 *g4 = reinterpret_cast<const int4 *>(mat[0].gidx);
+#pragma unroll
+        for (int u = 0; u < kStageBatch; u++) {
+            const int j4 = u * (NW * 64) + tid;
+            gi[u] = j4 < n4 ? g4[j4] : make_int4(0, 0, 0, 0);
+        }
+    }
     if constexpr (DIRECT) {
         // this wave's 64 chunks of x, 1 KB per load instruction (whole cache lines); past the end the last
         // 16 bytes are re-read and zeroed below
@@ -336,8 +353,23 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
         for (int q = 0; q < NM; q++) {
             const MatOps &M = mat[q];
             float *xs = lds + q * xstride;
-            float p = stage_consume<NW>(M.wn != nullptr, in, 0, tid, xr[q], xs, xs + C * kChunkPad, 0.f);
-            p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
+            float p = 0.f;
+            if constexpr (GATHER) {
+                const int n4 = in >> 2;
+#pragma unroll
+                for (int u = 0; u < kStageBatch; u++) {
+                    const int j4 = u * (NW * 64) + tid;
+                    if (j4 < n4) { // element 4 j4 + e of x is input gi[u].e of the sorted rows
+                        xs[(gi[u].x >> 5) * kChunkPad + (gi[u].x & 31)] = xr[q].v[u].x;
+                        xs[(gi[u].y >> 5) * kChunkPad + (gi[u].y & 31)] = xr[q].v[u].y;
+                        xs[(gi[u].z >> 5) * kChunkPad + (gi[u].z & 31)] = xr[q].v[u].z;
+                        xs[(gi[u].w >> 5) * kChunkPad + (gi[u].w & 31)] = xr[q].v[u].w;
+                    }
+                }
+            } else {
+                p = stage_consume<NW>(M.wn != nullptr, in, 0, tid, xr[q], xs, xs + C * kChunkPad, 0.f);
+                p = stage_rest<NW>(M.x + (size_t)b * in, M.wn, in, xs, xs + C * kChunkPad, tid, p);
+            }
             if (q == 0) ssq = p;
         }
         if (norm) {
@@ -390,7 +422,17 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
                         x[q][4 * i + 2] = v.z;
                         x[q][4 * i + 3] = v.w;
                     }
-                    sx[q] = xs[C * kChunkPad + c];
+                    if constexpr (GATHER) {
+                        // the chunk's sum in the association the block-wide staging uses (fours, then the tree of
+                        // its three cross-lane adds), so that both forms of the operator give the same bits
+                        float s4[8];
+#pragma unroll
+                        for (int k = 0; k < 8; k++)
+                            s4[k] = (x[q][4 * k] + x[q][4 * k + 1]) + (x[q][4 * k + 2] + x[q][4 * k + 3]);
+                        sx[q] = ((s4[0] + s4[1]) + (s4[2] + s4[3])) + ((s4[7] + s4[6]) + (s4[5] + s4[4]));
+                    } else {
+                        sx[q] = xs[C * kChunkPad + c];
+                    }
                 } else {
 #pragma unroll
                     for (int i = 0; i < 32; i++) x[q][i] = 0.f;
@@ -570,23 +612,25 @@ static long plan_cost(const Q4Launch &L, int NWK, int S, int P, bool pair) {
     return (long)per_cu * NW * tiles * P;
 }
 
-template <int G, int NWK, int S, bool PAIR, int MODE, int P = (PAIR ? 2 : 4)>
+template <int G, int NWK, int S, bool PAIR, int MODE, int P = (PAIR ? 2 : 4), bool GATHER = false>
 int launch_s(Q4Launch &L, hipStream_t stream) {
     constexpr int NW = NWK * S;
     constexpr int TR = P * S;
     const int C = L.in / 32;
     const size_t lds = MODE == 2 ? (size_t)NW * 64 * kChunkPad * sizeof(float)
                                  : (size_t)(C * kChunkPad + C) * sizeof(float) * (PAIR ? 2 : 1);
+    if (GATHER && L.in > NW * 64 * 4 * kStageBatch)
+        return l2_fail(L2_ERR_ARG, "q4 matvec (gathering): in=%d is more than one staging batch of %d waves", L.in, NW);
     if (lds + 8 * 1024 > 160 * 1024) return l2_fail(L2_ERR_ARG, "q4 matvec: in=%d needs %zu B of LDS", L.in, lds);
     int total = 0;
     const int rpb = plan_rows(L, NW, TR, lds, PAIR, &total);
     L.rows_per_block = rpb;
     for (int i = 0; i < L.n_mats; i++) L.m[i].row_blocks = (L.m[i].out + rpb - 1) / rpb;
-    auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE, P>;
+    auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE, P, GATHER>;
     if (g_q4_name.armed) {
         g_q4_name.armed = false;
-        snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_stream_kernel<%d, %d, %d, %s, %d, %d>", G, NWK, S,
-                 PAIR ? "true" : "false", MODE, P);
+        snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_stream_kernel<%d, %d, %d, %s, %d, %d%s>", G, NWK, S,
+                 PAIR ? "true" : "false", MODE, P, GATHER ? ", true" : "");
         g_q4_name.grid = total, g_q4_name.block = NW * 64, g_q4_name.rows_per_block = rpb, g_q4_name.lds = lds;
         return L2_OK;
     }
@@ -619,6 +663,13 @@ int launch_sg(Q4Launch &L, hipStream_t stream) {
                 return launch_s<G, 3, 4, false, MODE>(L, stream);
             case 7: return launch_s<G, 7, 2, false, MODE, 3>(L, stream);
             case 9: case 10: case 11: case 12: case 13: case 14: return launch_s<G, 14, 1, false, MODE>(L, stream);
+        }
+    } else if (MODE == 0 && !L.pair && L.n_mats == 1 && L.m[0].gidx) {
+        if constexpr (MODE == 0) switch (nwk) { // the gathering form, where one staging batch covers the vector
+            case 1: return launch_s<G, 1, 4, false, 0, 4, true>(L, stream);
+            case 2: return launch_s<G, 2, 4, false, 0, 2, true>(L, stream);
+            case 3: return launch_s<G, 3, 4, false, 0, 4, true>(L, stream);
+            case 4: return launch_s<G, 4, 4, false, 0, 2, true>(L, stream);
         }
     } else if (!L.pair) {
         switch (nwk) {
@@ -658,7 +709,7 @@ int q4_stream_launch(Q4Launch &L, hipStream_t stream) {
     // 8192: 11.6 -> 12.3, 4096 equal within the model.  The per-wave form is taken where it won: 3 and 7 waves
     // per row, and inputs too long to stage block-wide beside a second block.
     const int nwk = (L.in / 32 + 63) / 64;
-    const bool direct = fp32_form && !L.pair && L.n_mats == 1 && L.m[0].wn == nullptr &&
+    const bool direct = fp32_form && !L.pair && L.n_mats == 1 && L.m[0].wn == nullptr && L.m[0].gidx == nullptr &&
                         (L.in > 16384 || nwk == 3 || nwk == 7);
     if (direct) {
         switch (L.group_size) {
@@ -680,6 +731,20 @@ int q4_stream_launch(Q4Launch &L, hipStream_t stream) {
         }
     }
     return l2_fail(L2_ERR_ARG, "q4 matvec: group size %d (32, 64 or 128)", L.group_size);
+}
+
+static bool fp32_stream_form() {
+    static const bool yes = []() {
+        const char *v = getenv("L2_Q4_IMPL");
+        return !(v && (!strcmp(v, "idot") || !strcmp(v, "tile")));
+    }();
+    return yes;
+}
+
+bool q4_gathers_in_kernel(const Q4Launch &L) {
+    const int nwk = (L.in / 32 + 63) / 64;
+    return fp32_stream_form() && !L.pair && L.n_mats == 1 && L.m[0].wn == nullptr && nwk <= 4 && L.in % 4 == 0 &&
+           q4_stream_supports(L);
 }
 
 bool q4_stream_supports(const Q4Launch &L) {

@@ -100,7 +100,9 @@ struct Q4Mat {
     const uint4 *qweight;
     const int32_t *qzeros;
     const float *scales;
-    const float *x;  // input already in this layer's g_index order: [B][in]
+    const float *x;  // input already in this layer's g_index order: [B][in] (in its natural order if gidx is set)
+    const int32_t *gidx; // null, or the INVERSE of this layer's g_index: x is in its natural order and the kernel puts
+                         // x[b][i] where input gidx[i] of the sorted rows is read (one matrix, no rmsnorm)
     const float *wn; // rmsnorm weights in the same order, or null: x is used as it is
     float *y;        // [B][out]
     int out;
@@ -159,6 +161,9 @@ int q4_matvec_launch(Q4Launch &L, hipStream_t stream);
 // The two forms of the kernel behind q4_matvec_launch.
 int q4_stream_launch(Q4Launch &L, hipStream_t stream);
 bool q4_stream_supports(const Q4Launch &L);
+// Whether q4_matvec_launch would apply the act-order permutation itself for this launch if m[0].gidx were set (one
+// matrix, no rmsnorm, the default fp32 streaming form, rows of at most four waves); otherwise the caller gathers.
+bool q4_gathers_in_kernel(const Q4Launch &L);
 
 // ---- prefill chunks through the matrix cores ---------------------------------
 
