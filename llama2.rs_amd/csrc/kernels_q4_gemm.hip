@@ -657,12 +657,16 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     const int NB = B > 32 ? 2 : 1;
     const int TN = 32 * NB;
     const int t_tiles = (B + TN - 1) / TN;
-    // K slices: as many as keep the grid within one round of 2 blocks per CU, whole groups per slice, at most 8
+    // K slices: as many as keep the grid within one round of 2 blocks per CU, whole groups per slice, at most 4.
+    // (Up to 8 fill the chip when a launch runs alone, but every slice is a partial tile that the consumer reads
+    // back, and with two chunks of a prompt in flight the other chunk's kernels take the free slots: at most 4
+    // measured 34.4 k against 32.7 k tok/s on the 7B prompt, 19.9 k against 19.5 k on 13B, no change on 70B, and
+    // 25.1 k against 24.6 k with a single chunk in flight.)
     // K step: 128 where a group is at least that long (half the block barriers per k), else 64
     constexpr int KSTEP = G >= 128 ? 128 : 64;
     const int n_grp = (L.in / KSTEP) / (G / KSTEP > 0 ? G / KSTEP : 1);
     int KS = (2 * cu_count()) / (total * t_tiles); // all blocks resident at once: two per CU
-    if (KS > 8) KS = 8;
+    if (KS > 4) KS = 4;
     if (KS > n_grp / 2) KS = n_grp / 2; // slices start on even groups
     if (KS < 1) KS = 1;
     while (KS > 1 && (size_t)KS * B * rows > ws_floats) KS--;
