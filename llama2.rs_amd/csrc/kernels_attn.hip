@@ -821,225 +821,174 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(float *__restrict__ o
     }
 }
 
-// Chunk attention on the matrix cores, all in fp32 (v_mfma_f32_32x32x2_f32), for the prefill mode that
-// hands fp16 activations to the next GEMM.  Same function as attn_prefill_kernel (src/models.rs:131-176,
-// causal per query over the cache rows 0..pos).
-//
-// A block of 8 waves owns 32 columns of one kv head: column n = (query ct*32/QG + n/QG, head kvh*QG + n%QG).
-// Wave w takes the key tiles w, w+8, ... of 32 cache rows each and keeps a running (m, l, O) of its own;
-// the block merges the eight at the end.  Per tile, with lane = (n = lane%32, h = lane/32):
-//   S^T = K Q^T      A: lane (key n, h) holds K[key][64h + s], B: lane (column n, h) holds Q[n][64h + s]
-//                    (the contraction index of MFMA step s and half h is d = 64h + s), 64 steps.  K reaches
-//                    that layout through the wave's LDS tile: loaded lane-per-row-half, a load instruction
-//                    touches 64 cache lines and the address unit becomes the bottleneck.
-//   C layout         lane (column n, h), register r -> key (r/4)*8 + 4h + r%4: a lane holds 16 scores of
-//                    ITS column, so the running maximum and sum are per-lane work plus one exchange
-//                    between the two halves.
-//   O^T += V^T P^T   step s, half h contracts over key (s/4)*8 + 4h + s%4, which is the lane's own
-//                    register s of P: the B operand needs no data movement.  A: lane (d-row n, h) reads
-//                    V[key][32*mt + n] from the wave's LDS tile; 4 tiles of 32 d, 16 steps each.
-template <int QG>
-__global__ __launch_bounds__(512) void attn_prefill_mfma_kernel(_Float16 *__restrict__ out_h, const float *__restrict__ q,
-                                                                 const float *__restrict__ kc, const float *__restrict__ vc,
-                                                                 const int32_t *__restrict__ pos,
-                                                                 const int32_t *__restrict__ scatter, int n_heads,
-                                                                 int n_kv_heads, int B, int max_pos) {
-    constexpr int HS = 128, NWV = 8, TK = 32, QPT = 32 / QG;
-    constexpr int kQRow = 33;      // floats per d-row of the transposed Q tile
-    constexpr int kVRow = HS + 4;  // floats per key row of a staged V tile
-    typedef float v16f __attribute__((ext_vector_type(16)));
-    extern __shared__ float smem[];
-    float *qst = smem;                                  // [HS][kQRow]: Q^T of the block's 32 columns
-    __shared__ float m_s[NWV][32], l_s[NWV][32];
+// Chunk attention on the matrix cores, all in fp32 (v_mfma_f32_16x16x4_f32), for the prefill mode that hands fp16
+// activations to the next GEMM.  Same function as attn_prefill_kernel (src/models.rs:131-176, causal per query over
+// the cache rows 0..pos), in the layout of attn_decode_mfma_kernel: a block owns 16 columns of one kv head, column
+// n = (query ct*16/QG + n/QG, head kvh*QG + n%QG), its NWV waves take the tiles of 16 cache rows w, w + NWV, ...
+// and merge through LDS at the end.  With lane = (i = lane % 16, kb = lane / 16):
+//   S^T = K Q^T      A: lane (row i, kb) holds K[t][16 m + 4 kb + e] -- what a 16-byte load of the cache row leaves
+//                    in the lane; B: lane (column i, kb) holds Q[column][16 m + 4 kb + e], eight 16-byte loads of
+//                    the query's row, kept for the whole kernel.  Nothing passes through LDS on the way.
+//   C layout         lane (column j, kb), register r -> row 4 kb + r: the lane masks the rows behind ITS column's
+//                    position (causal per query); the four lanes of a column share its running maximum.
+//   O^T += V^T P^T   contracts over the lane's own registers of P; A is a 16-byte load of the V row as it stands.
+// 128 tokens of a 32-head model are 256 blocks, one per compute unit.  (A form on 32 columns and tiles of 32 rows,
+// v_mfma_f32_32x32x2_f32 with K and V turned through LDS, had half the blocks and took 16 to 31 us per chunk of a
+// 512-token prompt where this one takes 11 to 19.)
+template <int QG, int NWV>
+__global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1)
+void attn_prefill_mfma16_kernel(_Float16 *__restrict__ out_h, const float *__restrict__ q, const float *__restrict__ kc,
+                                const float *__restrict__ vc, const int32_t *__restrict__ pos,
+                                const int32_t *__restrict__ scatter, int n_heads, int n_kv_heads, int B, int max_pos) {
+    constexpr int NT = NWV * 64, TK = 16, HS = 128, HALF = 64, NC = 16, QPT = NC / QG;
+    __shared__ __align__(16) float comb[NWV][NC][kCombRow];
     const int kvh = blockIdx.x, ct = blockIdx.y;
     const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n = lane & 31, h = lane >> 5;
-    float *vs = smem + HS * kQRow + wave * (TK * kVRow); // this wave's V tile, later its partial O^T [HS][32]
-
-    const float scale = 1.44269504088896340736f / sqrtf((float)HS);
+    const int li = lane & 15, kb = lane >> 4;
     const uint32_t row_bytes = (uint32_t)kv_dim * 4u;
-    const int last_row = max_pos; // the last cache row written: loads clamp to it and wait for nothing
+    const uint32_t k_lane = (uint32_t)(kvh * HS + 4 * kb) * 4u; // + 64 m bytes
+    const uint32_t v_lane = (uint32_t)(kvh * HS + 4 * li) * 4u; // + 256 bytes for the second half of d
 
-    // K and V: the tile row by row, 16 bytes per lane and load (whole cache lines per instruction).  Rows past
-    // the end re-read the last row (masked below), so the loads are unconditional.
-    float4 kr[16], vr[16];
-    auto fetch_k = [&](int kt) { // row by row like V: 32 lanes read one row's 512 bytes
+    struct Tile {
+        float4 k[8]; // k[m]: K[t = li][16 m + 4 kb ..]
+        float4 v[8]; // v[2 r + half]: V[t = 4 kb + r][64 half + 4 li ..]
+    };
+    // Unconditional loads: rows past the last one written re-read it (masked below).
+    auto fetch = [&](int tile, Tile &d) {
+        const int tb = tile * TK;
+        const uint32_t ko = __umul24(min(tb + li, max_pos), row_bytes) + k_lane;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int f = i * 64 + lane;
-            const int tk = min(kt * TK + (f >> 5), last_row);
-            kr[i] = ld_at<float4>(kc, __umul24(tk, row_bytes) + (uint32_t)(kvh * HS + 4 * (f & 31)) * 4u);
+        for (int m = 0; m < 8; m++) d.k[m] = ld_at<float4>(kc, ko + 64u * m);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint32_t vo = __umul24(min(tb + 4 * kb + r, max_pos), row_bytes) + v_lane;
+            d.v[2 * r] = ld_at<float4>(vc, vo);
+            d.v[2 * r + 1] = ld_at<float4>(vc, vo + 256u);
         }
     };
-    auto fetch_v = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int f = i * 64 + lane;
-            const int tv = min(kt * TK + (f >> 5), last_row);
-            vr[i] = ld_at<float4>(vc, __umul24(tv, row_bytes) + (uint32_t)(kvh * HS + 4 * (f & 31)) * 4u);
-        }
-    };
-    fetch_k(wave);
-    fetch_v(wave);
-    __builtin_amdgcn_sched_barrier(0);
-    // positions of the 32 columns; the block's tiles end with the last row any of them sees
-    const int my_qi = ct * QPT + n / QG;
+    // this lane's column: its query, its position, its B operands
+    const int my_qi = ct * QPT + li / QG;
     const int my_pos = my_qi < B ? pos[my_qi] : -1;
-    int t_end = my_pos + 1;
+    const float *qrow = q + (size_t)min(my_qi, B - 1) * dim + (size_t)(kvh * QG + li % QG) * HS + 4 * kb;
+    float4 qf[8];
 #pragma unroll
-    for (int off = 16; off > 0; off >>= 1) t_end = max(t_end, __shfl_xor(t_end, off));
+    for (int m = 0; m < 8; m++) qf[m] = *reinterpret_cast<const float4 *>(qrow + 16 * m);
+    Tile ta, tb2;
+    fetch(wave, ta);
+    fetch(wave + NWV, tb2);
+    __builtin_amdgcn_sched_barrier(0);
+    int t_end = my_pos + 1; // the block's tiles end with the last row any of its columns sees
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) t_end = max(t_end, __shfl_xor(t_end, off));
     t_end = __builtin_amdgcn_readfirstlane(t_end);
-    const int n_kt = (t_end + TK - 1) / TK;
+    const int n_tiles = (t_end + TK - 1) / TK;
 
-    {   // Q^T of the 32 columns: all eight loads of a thread in flight, then the LDS writes
-        float qreg[8];
+    float m_run = kNoScore, l = 0.f;
+    v4f acc[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int idx = u * 512 + tid;
-            const int col = idx >> 7, d = idx & 127;
-            const int qi = min(ct * QPT + col / QG, B - 1);
-            qreg[u] = q[(size_t)qi * dim + (kvh * QG + col % QG) * HS + d];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int idx = u * 512 + tid;
-            qst[(idx & 127) * kQRow + (idx >> 7)] = qreg[u];
-        }
-    }
-    __syncthreads();
+    for (int c = 0; c < 8; c++) acc[c] = v4f{0.f, 0.f, 0.f, 0.f};
+    const float scale = 1.44269504088896340736f / sqrtf((float)HS); // log2(e) / sqrt(head_size), src/models.rs:154
 
-    float m = kNoScore, l = 0.f;
-    v16f o[4];
+    auto tile_math = [&](int tile, Tile &d) __attribute__((always_inline)) {
+        const int tb = tile * TK;
+        v4f s0 = v4f{0.f, 0.f, 0.f, 0.f}, s1 = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o[mt][r] = 0.f;
-
-    for (int kt = wave; kt < n_kt; kt += NWV) {
-        const int t0 = kt * TK;
-        v16f sacc;
-#pragma unroll
-        for (int r = 0; r < 16; r++) sacc[r] = 0.f;
-        // the Q operands of steps 4i+4..4i+7 are read from LDS while the MFMAs of steps 4i..4i+3 run
-        // K: the tile as loaded (row-wise, whole cache lines per load) -> the wave's LDS tile -> the A-operand
-        // layout (lane (key n, h) holds d = 64h .. 64h + 63); the next tile's keys go out meanwhile
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int f = i * 64 + lane;
-            *reinterpret_cast<float4 *>(&vs[(f >> 5) * kVRow + 4 * (f & 31)]) = kr[i];
+        for (int m = 0; m < 8; m += 2) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].x, qf[m].x, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].x, qf[m + 1].x, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].y, qf[m].y, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].y, qf[m + 1].y, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].z, qf[m].z, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].z, qf[m + 1].z, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m].w, qf[m].w, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(d.k[m + 1].w, qf[m + 1].w, s1, 0, 0, 0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        fetch_k(kt + NWV);
-        __builtin_amdgcn_sched_barrier(0);
-        float qv[2][4];
-        float4 ka[2];
+        float sc[4], p[4];
+        float mx = kNoScore;
 #pragma unroll
-        for (int e = 0; e < 4; e++) qv[0][e] = qst[(64 * h + e) * kQRow + n];
-        ka[0] = *reinterpret_cast<const float4 *>(&vs[n * kVRow + 64 * h]);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const float kk[4] = {ka[i & 1].x, ka[i & 1].y, ka[i & 1].z, ka[i & 1].w};
-            if (i + 1 < 16) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) qv[(i + 1) & 1][e] = qst[(64 * h + 4 * (i + 1) + e) * kQRow + n];
-                ka[(i + 1) & 1] = *reinterpret_cast<const float4 *>(&vs[n * kVRow + 64 * h + 4 * (i + 1)]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int e = 0; e < 4; e++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[e], qv[i & 1][e], sacc, 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // the V tile into the wave's own LDS region (the wave's LDS accesses execute in order)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int f = i * 64 + lane;
-            *reinterpret_cast<float4 *>(&vs[(f >> 5) * kVRow + 4 * (f & 31)]) = vr[i];
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        fetch_v(kt + NWV);
-        __builtin_amdgcn_sched_barrier(0);
-        // scores of this lane's column, running maximum shared by the two halves of the column
-        float sc[16];
-        float mx = m;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int key = t0 + (r >> 2) * 8 + 4 * h + (r & 3);
-            sc[r] = key <= my_pos ? sacc[r] * scale : kNoScore;
+        for (int r = 0; r < 4; r++) {
+            const bool valid = tb + 4 * kb + r <= my_pos; // causal: this column's query sees rows 0..pos
+            sc[r] = valid ? (s0[r] + s1[r]) * scale : kNoScore;
             mx = fmaxf(mx, sc[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        if (__any(mx > m)) {
-            const float c = exp2_fast(m - mx);
+        if (__any(mx > m_run)) { // some column's maximum moves: agree on it among the column's four lanes, rescale
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            const float c = exp2_fast(m_run - m_new);
             l *= c;
 #pragma unroll
-            for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[mt][r] *= c;
-            m = mx;
+            for (int cc = 0; cc < 8; cc++) acc[cc] *= c;
+            m_run = m_new;
         }
-        float pr[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int key = t0 + (r >> 2) * 8 + 4 * h + (r & 3);
-            pr[r] = key <= my_pos ? exp2_fast(sc[r] - m) : 0.f;
-            l += pr[r];
+        for (int r = 0; r < 4; r++) {
+            const bool valid = tb + 4 * kb + r <= my_pos;
+            p[r] = valid ? exp2_fast(sc[r] - m_run) : 0.f;
+            l += p[r];
         }
-        // likewise the V operands: those of step st + 1 are read while the four MFMAs of step st run
-        float vv[2][4];
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++) vv[0][mt] = vs[(4 * h) * kVRow + 32 * mt + n];
-#pragma unroll
-        for (int st = 0; st < 16; st++) {
-            if (st + 1 < 16) {
-                const int key = ((st + 1) >> 2) * 8 + 4 * h + ((st + 1) & 3);
-#pragma unroll
-                for (int mt = 0; mt < 4; mt++) vv[(st + 1) & 1][mt] = vs[key * kVRow + 32 * mt + n];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int mt = 0; mt < 4; mt++)
-                o[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[st & 1][mt], pr[st], o[mt], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+        for (int r = 0; r < 4; r++) {
+            const float4 v0 = d.v[2 * r], v1 = d.v[2 * r + 1];
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.x, p[r], acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.y, p[r], acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.z, p[r], acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(v0.w, p[r], acc[3], 0, 0, 0);
+            acc[4] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.x, p[r], acc[4], 0, 0, 0);
+            acc[5] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.y, p[r], acc[5], 0, 0, 0);
+            acc[6] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.z, p[r], acc[6], 0, 0, 0);
+            acc[7] = __builtin_amdgcn_mfma_f32_16x16x4f32(v1.w, p[r], acc[7], 0, 0, 0);
+        }
+    };
+    // two buffers, each refilled right after its tile is done when the wave has a further tile for it (uniform)
+    for (int tile = wave; tile < n_tiles; tile += 2 * NWV) {
+        tile_math(tile, ta);
+        if (tile + 2 * NWV < n_tiles) fetch(tile + 2 * NWV, ta);
+        if (tile + NWV < n_tiles) {
+            tile_math(tile + NWV, tb2);
+            if (tile + 3 * NWV < n_tiles) fetch(tile + 3 * NWV, tb2);
         }
     }
 
-    // this wave's (m, l, O^T) -> LDS; O^T [d][column] over the wave's V region
+    // this wave's (m, l, O) -> LDS: lane (column j, kb), accumulators 0..3, register r are d = 16 kb + 4 r + 0..3,
+    // accumulators 4..7 the same 64 further on
+    l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    if (h == 0) {
-        m_s[wave][n] = m;
-        l_s[wave][n] = l;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        *reinterpret_cast<float4 *>(&comb[wave][li][16 * kb + 4 * r]) = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+        *reinterpret_cast<float4 *>(&comb[wave][li][HALF + 16 * kb + 4 * r]) =
+            make_float4(acc[4][r], acc[5][r], acc[6][r], acc[7][r]);
     }
-#pragma unroll
-    for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) vs[(32 * mt + (r >> 2) * 8 + 4 * h + (r & 3)) * 32 + n] = o[mt][r];
+    if (kb == 0) {
+        comb[wave][li][HS] = m_run;
+        comb[wave][li][HS + 1] = l;
+    }
     __syncthreads();
-    const float *part = smem + HS * kQRow;
-    // a thread's column is the same in all eight passes; its scatter targets are fetched together
-    const int col = tid & 31;
-    const int qi = ct * QPT + col / QG;
-    int dst[8];
+    // merge the waves; a thread owns 8 consecutive d of one column, so that what it stores is one 16-byte piece of
+    // the fp16 pair-interleaved row when the consumer's order keeps those 8 together, and 8 two-byte stores otherwise
+    constexpr int NP = NC * HS / NT; // outputs per thread
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-        const int i = (kvh * QG + col % QG) * HS + u * 16 + (tid >> 5);
-        dst[u] = scatter ? scatter[i] : i;
-    }
-    if (qi >= B) return;
+    for (int u = 0; u < NP; u++) {
+        const int idx = tid + u * NT;
+        const int j = idx >> 7, d = idx & 127;
+        const int qi = ct * QPT + j / QG;
+        float M = comb[0][j][HS];
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-        const int d = u * 16 + (tid >> 5);
-        float M = m_s[0][col];
-#pragma unroll
-        for (int w = 1; w < NWV; w++) M = fmaxf(M, m_s[w][col]);
-        float num = 0.f, den = 0.f;
+        for (int w = 1; w < NWV; w++) M = fmaxf(M, comb[w][j][HS]);
+        float nu = 0.f, de = 0.f;
 #pragma unroll
         for (int w = 0; w < NWV; w++) {
-            const float e = exp2_fast(m_s[w][col] - M);
-            num = fmaf(e, part[w * (TK * kVRow) + d * 32 + col], num);
-            den = fmaf(e, l_s[w][col], den);
+            const float e = exp2_fast(comb[w][j][HS] - M);
+            nu = fmaf(e, comb[w][j][d], nu);
+            de = fmaf(e, comb[w][j][HS + 1], de);
         }
-        out_h[(size_t)qi * dim + h16_slot(dst[u])] = (_Float16)(num / den); // the order the next GEMM reads
+        if (qi < B) {
+            const int i = (kvh * QG + j % QG) * HS + d;
+            const int dst = scatter ? scatter[i] : i;
+            out_h[(size_t)qi * dim + h16_slot(dst)] = (_Float16)(nu / de); // the order the next GEMM reads
+        }
     }
 }
 
@@ -1138,21 +1087,13 @@ int attention_launch(float *out, void *out_f16, const float *q, const float *kca
     const int qg = n_heads / n_kv_heads;
     if (qg != 1 && qg != 2 && qg != 4 && qg != 8)
         return l2_fail(L2_ERR_ARG, "attention: %d query heads per kv head (1, 2, 4 or 8)", qg);
-    if (out_f16) { // the matrix-core form: 32 columns (queries x heads of the group) per block
-        constexpr size_t lds = (size_t)(128 * 33 + 8 * 32 * 132) * sizeof(float);
-        dim3 grid(n_kv_heads, (B * qg + 31) / 32), block(512);
-        auto launch = [&](auto kern) {
-            static LdsLimit limit; // per instantiation (the lambda is generic: one body per kernel)
-            L2_TRY(limit.ensure(reinterpret_cast<const void *>(kern), lds));
-            hipLaunchKernelGGL(kern, grid, block, lds, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads,
-                               n_kv_heads, B, max_pos);
-            return (int)L2_OK;
-        };
+    if (out_f16) { // the matrix-core form: 16 columns (queries x heads of the group) per block
+        dim3 grid(n_kv_heads, (B * qg + 15) / 16), block(256);
         switch (qg) {
-            case 1: L2_TRY(launch(attn_prefill_mfma_kernel<1>)); break;
-            case 2: L2_TRY(launch(attn_prefill_mfma_kernel<2>)); break;
-            case 4: L2_TRY(launch(attn_prefill_mfma_kernel<4>)); break;
-            default: L2_TRY(launch(attn_prefill_mfma_kernel<8>)); break;
+            case 1: hipLaunchKernelGGL((attn_prefill_mfma16_kernel<1, 4>), grid, block, 0, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B, max_pos); break;
+            case 2: hipLaunchKernelGGL((attn_prefill_mfma16_kernel<2, 4>), grid, block, 0, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B, max_pos); break;
+            case 4: hipLaunchKernelGGL((attn_prefill_mfma16_kernel<4, 4>), grid, block, 0, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B, max_pos); break;
+            default: hipLaunchKernelGGL((attn_prefill_mfma16_kernel<8, 4>), grid, block, 0, st, (_Float16 *)out_f16, q, kcache_l, vcache_l, pos, scatter, n_heads, n_kv_heads, B, max_pos); break;
         }
         L2_HIP(hipGetLastError());
         return L2_OK;
