@@ -629,8 +629,8 @@ int launch_s(Q4Launch &L, hipStream_t stream) {
     auto kern = q4_stream_kernel<G, NWK, S, PAIR, MODE, P, GATHER>;
     if (g_q4_name.armed) {
         g_q4_name.armed = false;
-        snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_stream_kernel<%d, %d, %d, %s, %d, %d%s>", G, NWK, S,
-                 PAIR ? "true" : "false", MODE, P, GATHER ? ", true" : "");
+        snprintf(g_q4_name.buf, (size_t)g_q4_name.cap, "q4_stream_kernel<%d, %d, %d, %s, %d, %d, %s>", G, NWK, S,
+                 PAIR ? "true" : "false", MODE, P, GATHER ? "true" : "false");
         g_q4_name.grid = total, g_q4_name.block = NW * 64, g_q4_name.rows_per_block = rpb, g_q4_name.lds = lds;
         return L2_OK;
     }
