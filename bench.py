@@ -319,7 +319,7 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool, c
 
     reps, spread = 5, []
 
-    def run(mode):
+    def run(mode, chunk=chunk):
         m.set_prefill_mode(mode)
         m.reset()
         m.prefill_chunks(np.concatenate([[1], prompt[:n - 1]]).astype(np.int32), 0, chunk)   # untimed: the whole prompt once
@@ -339,9 +339,23 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool, c
         spread.append((times[0], times[-1]))
         return times[len(times) // 2]
 
+    out = {}
+    if chunk < n:
+        # The same prompt as ONE pass of n tokens (the reference takes the longest prefill it was compiled with,
+        # src/inference.rs:77-125): reported beside the stated chunking, never instead of it.
+        t_one = run(_lib.PREFILL_MFMA, n)
+        ids_one, _ = m.decode_bench(int(prompt[-1]), n, K)
+        spread_one = spread.pop()
     t_mfma = run(_lib.PREFILL_MFMA)
     ids, ms_dec = m.decode_bench(int(prompt[-1]), n, K)
-    out = {}
+    if chunk < n:
+        tf_one = flops_per_token * (n / t_one) / 1e12
+        out["one_pass_of_the_prompt"] = {
+            "workload": f"the same {n}-token prompt as a single chunk of {n}", "value": round(n / t_one, 1), "unit": "tok/s",
+            "timing": f"median of {reps} (fastest {n / spread_one[0]:.0f}, slowest {n / spread_one[1]:.0f} tok/s)",
+            "roofline": {"bound": "mfma", "achieved": round(tf_one, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tf_one / MFMA_F16_PEAK_TFLOPS, 4)},
+            "greedy_tokens_same_as_after_the_chunked_prefill": f"{int(np.sum(np.cumprod(ids == ids_one)))}/{K}"}
     if compare_fp32:
         t_fp32 = run(_lib.PREFILL_FP32)
         ids32, _ = m.decode_bench(int(prompt[-1]), n, K)
@@ -387,6 +401,37 @@ def prefill_run(np, M: Loaded, n: int, chunk: int, K: int, compare_fp32: bool, c
     return out
 
 
+def vendor_gemm_run() -> dict:
+    """Context for the prefill figures, not a product path: what the vendor library's own fp16 GEMM (hipBLASLt
+    behind torch.matmul) reaches on the Llama-2-7B projection shapes with fp16 weights already in HBM, so without
+    any dequantisation, at the token counts the prefill uses."""
+    import torch
+    shapes = {"wq|wk|wv": (12288, 4096), "wo": (4096, 4096), "w1|w3": (22016, 4096), "w2": (4096, 11008)}
+    out = {"metric": "vendor fp16 GEMM on the 7B projection shapes (context)", "unit": "us per launch", "rows": {}}
+    for tokens in (128, 512):
+        total = 0.0
+        for name, (n_out, n_in) in shapes.items():
+            x = torch.randn(tokens, n_in, device="cuda", dtype=torch.float16)
+            ws = [torch.randn(n_out, n_in, device="cuda", dtype=torch.float16) for _ in range(6)]   # 6 copies: not L2-resident
+            for w in ws:
+                x @ w.t()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                for w in ws:
+                    x @ w.t()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 60
+            total += us
+            tf = 2.0 * tokens * n_in * n_out / us / 1e6
+            out["rows"][f"{name} x {tokens} tokens"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1),
+                                                         "frac_of_fp16_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
+        out["rows"][f"one layer x {tokens} tokens"] = {"us": round(total, 1)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -403,9 +448,11 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="decoded tokens of the CPU sample (0 = sized to ~15 s)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "matvec"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "matvec", "vendor-gemm"],
                     help="prefill: BASELINE config 2 alone (prompt in chunks through the dequant->fp16 MFMA GEMM, then decode); "
-                         "matvec: BASELINE config 0 alone (the standalone 4096x4096 group-128 matvec)")
+                         "matvec: BASELINE config 0 alone (the standalone 4096x4096 group-128 matvec); "
+                         "vendor-gemm: context only, the vendor library's plain fp16 GEMM (torch.matmul on fp16 weights, no "
+                         "dequantisation) on the 7B projection shapes at 128 and 512 tokens")
     ap.add_argument("--instances", type=int, default=64, help="matvec: distinct weight instances cycled through")
     ap.add_argument("--iters", type=int, default=2048, help="matvec: launches per timed run")
     ap.add_argument("--prompt-len", type=int, default=512)
@@ -441,6 +488,10 @@ def main() -> int:
                   "config": {"workload": r["workload"], "seed": 0}}
         result.update({k: v for k, v in r.items() if k not in result and k != "workload"})
         print(json.dumps(result))
+        return 0
+
+    if a.workload == "vendor-gemm":
+        print(json.dumps(vendor_gemm_run()))
         return 0
 
     M = Loaded(ops, a.model, a.group, a.layers, a.kv_prefill + max(W + K, 16 + 256) + 16, a.seed)

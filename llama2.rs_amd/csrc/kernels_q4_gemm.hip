@@ -101,7 +101,7 @@ constexpr int gemm_wr(int kstep) { return 256 / kstep; }
 constexpr int gemm_xp(int kstep) { return 128 / kstep; }
 
 template <int G, int NB, int KSTEP>
-__global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
+__global__ __launch_bounds__(256, NB > 2 ? 2 : 1) void q4_gemm_kernel(const Q4Launch L, const XhList xh_list, const float *__restrict__ ss,
                                                       float *__restrict__ ws, int KS, int partials) {
     constexpr int PW = kGemmPW, XP = gemm_xp(KSTEP), WR = gemm_wr(KSTEP);
     static_assert(PW % WR == 0 && PW % XP == 0, "ring slots are indexed by the position in the unrolled body");
@@ -139,14 +139,11 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
     const int ghalf = tid >> 7;
 
     f16v acc[NB];  // running result
-    f16v accg[NB]; // partial sum of the current group (SA only)
+    f16v accg[NB]; // partial sum of the current group (SA only): every K step starts it from zero
 #pragma unroll
     for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            acc[nb][i] = 0.f;
-            accg[nb][i] = 0.f;
-        }
+        for (int i = 0; i < 16; i++) acc[nb][i] = 0.f;
     constexpr int KPG = G / KSTEP > 0 ? G / KSTEP : 1; // K iterations per group
     // this block's slice of K, in whole groups
     const int ks = blockIdx.z;
@@ -315,8 +312,9 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
                 if (step + 1 < NSTEP) produce(step + 1, (step + 1) & 1);
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
-                    if (SA)
-                        accg[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[step & 1], bq[step & 1][nb], accg[nb], 0, 0, 0);
+                    if (SA) // a K step is one group: its first MFMA starts from zero, so the fold below clears nothing
+                        accg[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[step & 1], bq[step & 1][nb],
+                                                                          step == 0 ? f16v{} : accg[nb], 0, 0, 0);
                     else
                         acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[step & 1], bq[step & 1][nb], acc[nb], 0, 0, 0);
                 }
@@ -332,10 +330,8 @@ __global__ __launch_bounds__(256) void q4_gemm_kernel(const Q4Launch L, const Xh
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
+                        for (int e = 0; e < 4; e++)
                             acc[nb][4 * q + e] = fmaf(svv[e], accg[nb][4 * q + e], acc[nb][4 * q + e]);
-                            accg[nb][4 * q + e] = 0.f;
-                        }
                 }
                 if (u == PW - 1) store_gs(base / PW + 1, gs2), store_zs(base / PW + 1, zs2); // fetched at the round's first step
             }
@@ -651,10 +647,12 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
         rows += L.m[i].out;
     }
     const int B = L.batch;
-    // 64 tokens per block even for longer chunks: 128 would halve the weight traffic, but its 128
-    // accumulator registers leave one block per CU, and the K loop (a barrier every 64 k) then has nothing
-    // to overlap with (measured: w1|w3 of 7B at 128 tokens 73 us, at 2 x 64 tokens 52 us).
-    const int NB = B > 32 ? 2 : 1;
+    // Up to 255 tokens a wave takes 64 of them: with 128 a chunk of 128 tokens is too few blocks for the chip
+    // (w1|w3 of 7B: 172 blocks on 256 CUs; the launches of a 128-token chunk are 7 % slower that way).  From
+    // 256 tokens on a wave takes 128 (within 256 registers: two blocks per CU): every weight is dequantised
+    // once per 128 tokens instead of twice, and there are blocks enough whatever the tile (w1|w3 of 7B at 512
+    // tokens: 115 against 129 us).
+    const int NB = (G >= 64 && B >= 256) ? 4 : B > 32 ? 2 : 1;
     const int TN = 32 * NB;
     const int t_tiles = (B + TN - 1) / TN;
     // K slices: as many as keep the grid within one round of 2 blocks per CU, whole groups per slice, at most 4.
@@ -676,6 +674,14 @@ int launch_gemm_g(Q4Launch &L, const XhList &xh, const float *ss, float *ws, siz
     switch (NB) {
         case 1: hipLaunchKernelGGL((q4_gemm_kernel<G, 1, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS, ks_out != nullptr); break;
         case 2: hipLaunchKernelGGL((q4_gemm_kernel<G, 2, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS, ks_out != nullptr); break;
+        case 4:
+            if constexpr (G >= 64) {
+                static LdsLimit limit(48 * 1024);
+                L2_TRY(limit.ensure(reinterpret_cast<const void *>(q4_gemm_kernel<G, 4, KSTEP>), lds));
+                hipLaunchKernelGGL((q4_gemm_kernel<G, 4, KSTEP>), grid, block, lds, st, L, xh, ss, ws, KS, ks_out != nullptr);
+                break;
+            }
+            [[fallthrough]];
         default: return l2_fail(L2_ERR_ARG, "q4 gemm: token tile");
     }
     L2_HIP(hipGetLastError());

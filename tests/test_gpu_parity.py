@@ -719,10 +719,14 @@ def test_prefill_chunks_on_other_numbers_of_lanes(lanes):
     assert r.stdout.strip().endswith("BAD 0"), r.stdout[-500:]
 
 
+LONG_G128 = ck.Dims(dim=512, hidden_dim=768, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=260,
+                    seq_len=330, group_size=128)
+
+
 @pytest.mark.parametrize("dims,B", [(TINY_GQA, 5), (MID, 33), (MID, 128), (TINY, 37), (GQA8_G64, 5), (GQA8_G64, 64),
-                                    (GQA8_G64, 130)],
+                                    (GQA8_G64, 130), (LONG_G128, 256), (LONG_G128, 300)],
                          ids=["gqa_g128_b5", "g32_b33", "g32_b128", "mha_g64_b37", "gqa8_g64_b5", "gqa8_g64_b64",
-                              "gqa8_g64_b130"])
+                              "gqa8_g64_b130", "gqa_g128_b256", "gqa_g128_b300"])
 def test_mfma_prefill_operator_and_forward(ops, oracle, dims, B):
     """The dequant->fp16->MFMA form of QLinear::matvec<B> and of transformer<B> (B > 1)."""
     from llama2_rs import _lib

@@ -122,7 +122,7 @@ def test_70b_reduced_greedy_behind_4096_positions(ops, oracle, reduced_70b):
         assert nrel(v, vo[l, ctx:ctx + n]) < REL_FP32
 
 
-@pytest.mark.parametrize("B", [5, 64, 128, 130])
+@pytest.mark.parametrize("B", [5, 64, 128, 130, 256, 300])
 def test_70b_shapes_mfma_operator_group_64(ops, oracle, reduced_70b, B):
     """The dequant -> fp16 -> MFMA form of QLinear::matvec<B> at group 64 (K steps of 64, one group per
     step) on the 70B projections: rows of 8192 and of 28672 inputs, 8192, 1024 and 28672 outputs."""
@@ -196,51 +196,53 @@ def test_7b_wide_prefill_512_in_chunks_of_128_mfma(ops, oracle):
 
 def test_7b_full_depth_prefill_512_mfma_then_64_greedy(ops, oracle):
     """BASELINE config 2 at full depth: the Llama-2-7B architecture in full (32 layers), a 512-token random prompt
-    through l2_prefill_chunks (chunks of 128, dequant -> fp16 -> MFMA, two streams), then 64 greedy tokens, against
-    the oracle's fp32 prefill of the same prompt and its B=1 loop.  The fp16 rounding of every projection input
-    compounds over 32 layers: the last layer's cache rows are held to 2.5x the operator's 2e-3 (the bound of the
-    shallow whole-stack tests), the logits that follow the prompt to 2e-3, and the greedy tokens are compared one
-    by one; the first index at which they part, if any, is printed (fp16 rounding may flip a near-tie; a flip
-    within the first 8 tokens fails the test)."""
+    through l2_prefill_chunks (dequant -> fp16 -> MFMA; in chunks of 128 on two streams, and again as one pass of
+    512 tokens, which takes the 128-token wave tiles of the GEMM), then 64 greedy tokens, against the oracle's fp32
+    prefill of the same prompt and its B=1 loop.  The fp16 rounding of every projection input compounds over 32
+    layers: the last layer's cache rows are held to 2.5x the operator's 2e-3 (the bound of the shallow whole-stack
+    tests), the logits that follow the prompt to 2e-3, and the greedy tokens are compared one by one; the first
+    index at which they part, if any, is printed (fp16 rounding may flip a near-tie; a flip within the first 8
+    tokens fails the test)."""
     from llama2_rs import _lib
     dims = ops.preset("7B", 128)
     img = ops.synth_image(dims, 0)
-    n, chunk, n_greedy = 512, 128, 64
+    n, n_greedy = 512, 64
     m = ops.Model(img, dims, max_seq=n + n_greedy + 8)
     o = oracle.Model(img, dims, max_seq=n + n_greedy + 8)
     rng = np.random.default_rng(0)
     prompt = rng.integers(0, dims.vocab_size, size=n).astype(np.int32)
     toks = np.concatenate([[1], prompt[:-1]]).astype(np.int32)   # START-shifted, as prefill<A> feeds them
-    m.set_prefill_mode(_lib.PREFILL_MFMA)
-    m.reset()
-    m.prefill_chunks(toks, 0, chunk)
     o.new_state()
     for c0 in range(0, n, 64):   # the reference's ladder starts with chunks of 64 (src/inference.rs:78-85)
         o.transformer(toks[c0:c0 + 64], np.arange(c0, c0 + 64, dtype=np.int32))
     ko, vo = o.kv_cache()
-    errs = []
-    for l in (0, dims.n_layers // 2, dims.n_layers - 1):
-        k, v = m.read_kv(l, 0, n)
-        errs.append((l, nrel(k, ko[l, :n]), nrel(v, vo[l, :n])))
-    got = m.forward([int(prompt[-1])], [n])
     want = o.transformer([int(prompt[-1])], [n])
-    e_logits = nrel(got, want)
-    print(f"\ncfg2 full depth: cache rows (layer, k, v) {[(l, f'{a:.2e}', f'{b:.2e}') for l, a, b in errs]}, "
-          f"logits after the prompt {e_logits:.2e}")
     tok = oracle.argmax(want)
-    ids, _ = m.decode_bench(int(np.argmax(got)), n + 1, n_greedy - 1)
-    ids = np.concatenate([[int(np.argmax(got))], ids])
     ref = [tok]
     for pos in range(n + 1, n + n_greedy):
         tok = oracle.argmax(o.transformer([tok], [pos]))
         ref.append(tok)
     ref = np.asarray(ref)
-    same = int(np.sum(np.cumprod(ids == ref)))
-    print(f"cfg2 full depth: {same}/{n_greedy} greedy tokens identical to the CPU path"
-          + ("" if same == n_greedy else f"; they part at index {same}: GPU {ids[same]} CPU {ref[same]}"))
-    assert errs[-1][1] < 2.5 * REL_MFMA and errs[-1][2] < 2.5 * REL_MFMA, errs
-    assert e_logits < REL_MFMA, e_logits
-    assert same >= 8, (same, ids[:same + 1], ref[:same + 1])
+    m.set_prefill_mode(_lib.PREFILL_MFMA)
+    for chunk in (128, 512):
+        m.reset()
+        m.prefill_chunks(toks, 0, chunk)
+        errs = []
+        for l in (0, dims.n_layers // 2, dims.n_layers - 1):
+            k, v = m.read_kv(l, 0, n)
+            errs.append((l, nrel(k, ko[l, :n]), nrel(v, vo[l, :n])))
+        got = m.forward([int(prompt[-1])], [n])
+        e_logits = nrel(got, want)
+        print(f"\ncfg2 full depth, chunks of {chunk}: cache rows (layer, k, v) "
+              f"{[(l, f'{a:.2e}', f'{b:.2e}') for l, a, b in errs]}, logits after the prompt {e_logits:.2e}")
+        ids, _ = m.decode_bench(int(np.argmax(got)), n + 1, n_greedy - 1)
+        ids = np.concatenate([[int(np.argmax(got))], ids])
+        same = int(np.sum(np.cumprod(ids == ref)))
+        print(f"cfg2 full depth, chunks of {chunk}: {same}/{n_greedy} greedy tokens identical to the CPU path"
+              + ("" if same == n_greedy else f"; they part at index {same}: GPU {ids[same]} CPU {ref[same]}"))
+        assert errs[-1][1] < 2.5 * REL_MFMA and errs[-1][2] < 2.5 * REL_MFMA, (chunk, errs)
+        assert e_logits < REL_MFMA, (chunk, e_logits)
+        assert same >= 8, (chunk, same, ids[:same + 1], ref[:same + 1])
     m.close()
     o.close()
 
