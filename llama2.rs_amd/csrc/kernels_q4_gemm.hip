@@ -305,6 +305,9 @@ __global__ __launch_bounds__(256, NB > 2 ? 2 : 1) void q4_gemm_kernel(const Q4La
                 aq[slot] = dequant8<!SA>(wd[sw][j], dc, s16);
             };
             produce(0, 0);
+            // The wave that has its MFMAs to issue goes first on its SIMD; the other wave there is in its fold, its
+            // tile store or at its barrier (q|k|v at 512 tokens 68 -> 64 us, the other launches 1-4 %).
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int step = 0; step < NSTEP; step++) {
 #pragma unroll
@@ -320,6 +323,7 @@ __global__ __launch_bounds__(256, NB > 2 ? 2 : 1) void q4_gemm_kernel(const Q4La
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            __builtin_amdgcn_s_setprio(0);
             if (SA && (u + 1) % KPG == 0) {
                 // end of a group: fold its partial sum into the result with the fp32 scale of each row
                 const int gb = (base / PW) & 1;
