@@ -842,7 +842,8 @@ void attn_prefill_mfma16_kernel(_Float16 *__restrict__ out_h, const float *__res
                                 const int32_t *__restrict__ scatter, int n_heads, int n_kv_heads, int B, int max_pos) {
     constexpr int NT = NWV * 64, TK = 16, HS = 128, HALF = 64, NC = 16, QPT = NC / QG;
     __shared__ __align__(16) float comb[NWV][NC][kCombRow];
-    const int kvh = blockIdx.x, ct = blockIdx.y;
+    // the last columns of a chunk see the most cache rows: their blocks are dispatched first
+    const int kvh = blockIdx.x, ct = gridDim.y - 1 - blockIdx.y;
     const int dim = n_heads * HS, kv_dim = n_kv_heads * HS;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, kb = lane >> 4;
