@@ -629,14 +629,17 @@ _WIDE_7B = ck.Dims(dim=4096, hidden_dim=11008, n_layers=2, n_heads=32, n_kv_head
 @pytest.mark.parametrize("mode", ["mfma", "fp32"])
 @pytest.mark.parametrize("geom,n,chunk", [
     (_SMALL_QG2, 512, 128), (_SMALL_QG2, 300, 128), (_SMALL_QG2, 257, 64), (_SMALL_QG2, 40, 64), (_SMALL_QG2, 9, 2),
-    (GQA8_G64, 300, 128), (MID, 300, 128), (_WIDE_7B, 300, 128)],
+    (GQA8_G64, 300, 128), (MID, 300, 128), (_WIDE_7B, 300, 128),
+    (_SMALL_QG2, 700, 256), (GQA8_G64, 600, 256), (_WIDE_7B, 600, 256)],
     ids=["four_chunks", "short_last_chunk", "one_token_left", "one_short_chunk", "chunks_of_2",
-         "gqa8_g64_300_by_128", "qg4_g32_300_by_128", "7b_wide_300_by_128"])
+         "gqa8_g64_300_by_128", "qg4_g32_300_by_128", "7b_wide_300_by_128",
+         "three_chunks_of_256", "gqa8_g64_600_by_256", "7b_wide_600_by_256"])
 def test_prefill_chunks_equals_chunk_by_chunk(ops, geom, n, chunk, mode):
     """prefill<A> over a whole prompt (src/inference.rs:16-40) through l2_prefill_chunks, whose chunks overlap on
     two streams in the matrix-core mode, against the same chunks given to transformer<B> one by one: every cache
     row of every layer and the logits that follow, bit for bit (the kernels and their operands are the same).
-    Geometries: 2, 4 and 8 query heads per kv head, groups of 32, 64 and 128, and the 7B widths."""
+    Geometries: 2, 4 and 8 query heads per kv head, groups of 32, 64 and 128, and the 7B widths; chunks of 256
+    take the GEMM's 128-token wave tiles."""
     from llama2_rs import _lib
     from llama2_rs._lib import L2Error
     if geom is _WIDE_7B and mode == "fp32":
