@@ -328,8 +328,11 @@ int dense_launch(const DenseArgs &a0, hipStream_t st) {
     const int KI = ki <= 4 ? 4 : ki <= 8 ? 8 : ki <= 16 ? 16 : ki <= 20 ? 20 : 32;
     const int R = 32 / KI >= 1 ? 32 / KI : 1;
     a.n_pass = (ki + KI - 1) / KI;
-    // three blocks per CU (the registers allow three waves per SIMD), fewer when the rows run out
-    int blocks = (3 * 256 + a.batch - 1) / a.batch;
+    // One column (the classifier of a decode step): one block per CU -- 7B 93 -> 85 us, 13B 112 -> 103, 70B 172 ->
+    // 161 against three per CU, which the registers would allow and which stays the rule for several columns.
+    // Fewer when the rows run out.
+    const int per_cu = a.batch == 1 ? 1 : 3;
+    int blocks = (per_cu * cu_count() + a.batch - 1) / a.batch;
     const int need = (a.out + 4 * R - 1) / (4 * R);
     if (blocks > need) blocks = need;
     const size_t lds = (size_t)a.n_pass * KI * 64 * 16;

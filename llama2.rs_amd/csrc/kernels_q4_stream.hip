@@ -574,10 +574,11 @@ __global__ __launch_bounds__(NWK *S * 64) void q4_stream_kernel(const Q4Launch L
 }
 
 // Rows per block for a block of NW waves and tiles of TR rows: a whole number of rounds over the CUs, as
-// many blocks per CU as 16 waves and the LDS allow; every block gets the same number of rows; several
-// matrices round up separately and the grid stays within one round.
+// many blocks per CU as 16 waves and the LDS allow (one for a row pair); every block gets the same number of
+// rows; several matrices round up separately and the grid stays within one round.
 static int plan_rows(const Q4Launch &L, int NW, int TR, size_t lds, bool pair, int *total_out) {
     int per_cu = 16 / NW;
+    if (pair) per_cu = 1; // w1|w3: one block per CU measured faster than two (7B: 13.1 -> 12.4 us, 722 -> 733 tok/s)
     if (per_cu < 1) per_cu = 1;
     const int by_lds = (int)((150 * 1024) / (lds + 4 * 1024));
     if (per_cu > by_lds) per_cu = by_lds < 1 ? 1 : by_lds;
@@ -604,6 +605,7 @@ static long plan_cost(const Q4Launch &L, int NWK, int S, int P, bool pair) {
     const size_t lds = (size_t)(C * kChunkPad + C) * sizeof(float) * (pair ? 2 : 1);
     const int NW = NWK * S, TR = P * S;
     int per_cu = 16 / NW;
+    if (pair) per_cu = 1; // w1|w3: one block per CU measured faster than two (7B: 13.1 -> 12.4 us, 722 -> 733 tok/s)
     if (per_cu < 1) per_cu = 1;
     const int by_lds = (int)((150 * 1024) / (lds + 4 * 1024));
     if (per_cu > by_lds) per_cu = by_lds < 1 ? 1 : by_lds;
